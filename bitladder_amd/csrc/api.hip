@@ -1,0 +1,202 @@
+// C ABI of libbitdecode.so: argument validation, split choice, workspace carving, launches.
+// Host-side counterpart of csrc/bit_decode/decode_api.cpp:301-441 (decode) and :517-603 (pack)
+// in the reference; unsupported configurations return an error instead of silently doing nothing
+// (decode_api.cpp:190-202 leaves the output uninitialised there).
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <algorithm>
+
+#include "../../include/bitdecode.h"
+#include "kernels.h"
+#include "layout.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_quant(int bits, int gs, int dtype, int d) {
+    if (d != bitdecode::kHeadDim) return fail(BITDECODE_EUNSUPPORTED, "head_dim %d unsupported (only 128)", d);
+    if (bits != 2 && bits != 4) return fail(BITDECODE_EUNSUPPORTED, "num_bits %d unsupported (2 or 4)", bits);
+    if (gs != 32 && gs != 64 && gs != 128)
+        return fail(BITDECODE_EUNSUPPORTED, "group_size %d unsupported (32, 64 or 128)", gs);
+    if (dtype != BITDECODE_FP16 && dtype != BITDECODE_BF16)
+        return fail(BITDECODE_EUNSUPPORTED, "dtype %d unsupported (fp16=0, bf16=1)", dtype);
+    return 0;
+}
+
+int query_cus() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    return n;
+}
+
+// One wave handles one work unit (a 128-token packed chunk or a 32-token fp16 block) at a time and
+// a workgroup has 8 waves.  Pick the number of splits so that the whole grid is about one
+// workgroup per CU while every wave still gets at least one unit.
+int choose_splits(int b, int hk, int max_units, int num_cus) {
+    if (max_units <= 0) return 1;
+    const int heads = std::max(1, b * hk);
+    const int by_occupancy = std::max(1, (num_cus + heads - 1) / heads);
+    const int by_work = std::max(1, (max_units + 7) / 8);
+    int n = std::min(by_occupancy, by_work);
+    n = std::min(n, 256);
+    // drop splits that would be empty: ceil(units / n) units per split
+    const int ups = (max_units + n - 1) / n;
+    n = (max_units + ups - 1) / ups;
+    return std::max(1, n);
+}
+
+int units_of(int seqlen_k, int res_len) { return seqlen_k / bitdecode::kChunk + (res_len + 31) / 32; }
+
+}  // namespace
+
+extern "C" {
+
+int bitdecode_abi_version(void) { return BITDECODE_ABI_VERSION; }
+
+const char* bitdecode_last_error(void) { return g_err; }
+
+int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len, int32_t num_cus) {
+    if (num_cus <= 0) num_cus = query_cus();
+    return choose_splits(b, h_k, units_of(max_seqlen_k, max_res_len), num_cus);
+}
+
+size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
+    if (num_splits <= 1) return 0;
+    return static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 1) * sizeof(float);
+}
+
+int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
+    using namespace bitdecode;
+    if (!a) return fail(BITDECODE_EINVAL, "args is null");
+    if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
+    if (a->b < 0 || a->h_k <= 0 || a->n_tokens < 0) return fail(BITDECODE_EINVAL, "negative size");
+    if (a->n_tokens % kChunk) return fail(BITDECODE_EINVAL, "n_tokens %d is not a multiple of 128", a->n_tokens);
+    if (a->cache_tokens % kChunk || a->cache_tokens <= 0)
+        return fail(BITDECODE_EINVAL, "cache_tokens %d is not a positive multiple of 128", a->cache_tokens);
+    if (!a->dst_offsets) {
+        if (a->dst_offset < 0 || a->dst_offset % kChunk)
+            return fail(BITDECODE_EINVAL, "dst_offset %d is not a multiple of 128", a->dst_offset);
+        if (a->dst_offset + a->n_tokens > a->cache_tokens)
+            return fail(BITDECODE_EINVAL, "dst_offset %d + n_tokens %d exceeds cache capacity %d", a->dst_offset,
+                        a->n_tokens, a->cache_tokens);
+    } else if (a->n_tokens > a->cache_tokens) {
+        return fail(BITDECODE_EINVAL, "n_tokens %d exceeds cache capacity %d", a->n_tokens, a->cache_tokens);
+    }
+    if (a->n_tokens == 0 || a->b == 0) return BITDECODE_OK;
+    if (!a->k || !a->v || !a->k_pack || !a->k_params || !a->v_pack || !a->v_params)
+        return fail(BITDECODE_EINVAL, "null tensor pointer");
+    if (!aligned16(a->k) || !aligned16(a->v) || !aligned16(a->k_pack) || !aligned16(a->k_params) ||
+        !aligned16(a->v_pack) || !aligned16(a->v_params))
+        return fail(BITDECODE_EINVAL, "tensor pointers must be 16-byte aligned");
+    const int64_t strides[6] = {a->k_stride_b, a->k_stride_t, a->k_stride_h, a->v_stride_b, a->v_stride_t, a->v_stride_h};
+    for (int64_t s : strides)
+        if (s % 8) return fail(BITDECODE_EINVAL, "K/V strides must be multiples of 8 elements");
+
+    QpackParams P{};
+    P.k = static_cast<const uint16_t*>(a->k);
+    P.v = static_cast<const uint16_t*>(a->v);
+    P.k_sb = a->k_stride_b; P.k_st = a->k_stride_t; P.k_sh = a->k_stride_h;
+    P.v_sb = a->v_stride_b; P.v_st = a->v_stride_t; P.v_sh = a->v_stride_h;
+    P.k_pack = static_cast<uint8_t*>(a->k_pack);
+    P.k_params = static_cast<uint8_t*>(a->k_params);
+    P.v_pack = static_cast<uint8_t*>(a->v_pack);
+    P.v_params = static_cast<uint8_t*>(a->v_params);
+    P.kpack_bh = code_region_bytes(a->cache_tokens, a->bits);
+    P.vpack_bh = P.kpack_bh;
+    P.kparams_bh = k_param_region_bytes(a->cache_tokens, a->group_size);
+    P.vparams_bh = v_param_region_bytes(a->cache_tokens, a->group_size);
+    P.b = a->b; P.n_tokens = a->n_tokens; P.hk = a->h_k;
+    P.dst_offset = a->dst_offset;
+    P.dst_offsets = a->dst_offsets;
+    P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
+    hipError_t e = launch_qpack(P, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "qpack launch failed: %s", hipGetErrorString(e));
+    return BITDECODE_OK;
+}
+
+int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
+    using namespace bitdecode;
+    if (!a) return fail(BITDECODE_EINVAL, "args is null");
+    if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
+    if (a->b <= 0 || a->h <= 0 || a->h_k <= 0) return fail(BITDECODE_EINVAL, "batch and head counts must be positive");
+    if (a->h % a->h_k) return fail(BITDECODE_EINVAL, "h %d is not a multiple of h_k %d", a->h, a->h_k);
+    const int g = a->h / a->h_k;
+    if (g > kMaxGroupHeads)
+        return fail(BITDECODE_EUNSUPPORTED, "%d query heads per kv head unsupported (at most %d)", g, kMaxGroupHeads);
+    const int max_s = a->seqlens_k ? a->max_seqlen_k : a->seqlen_k;
+    const int max_r = a->res_lens ? a->max_res_len : a->res_len;
+    if (max_s < 0 || max_r < 0) return fail(BITDECODE_EINVAL, "negative length");
+    if (max_s % kChunk) return fail(BITDECODE_EINVAL, "packed length %d is not a multiple of 128", max_s);
+    if (max_s > a->cache_tokens) return fail(BITDECODE_EINVAL, "packed length %d exceeds cache capacity %d", max_s, a->cache_tokens);
+    if (max_s > 0 && (a->cache_tokens % kChunk)) return fail(BITDECODE_EINVAL, "cache_tokens must be a multiple of 128");
+    if (!a->q || !a->out) return fail(BITDECODE_EINVAL, "q/out is null");
+    if (max_s > 0 && (!a->k_pack || !a->k_params || !a->v_pack || !a->v_params))
+        return fail(BITDECODE_EINVAL, "null packed-cache pointer");
+    if (max_r > 0 && (!a->k_res || !a->v_res)) return fail(BITDECODE_EINVAL, "null residual pointer");
+    if (!aligned16(a->q) || !aligned16(a->k_pack) || !aligned16(a->k_params) || !aligned16(a->v_pack) ||
+        !aligned16(a->v_params) || !aligned16(a->k_res) || !aligned16(a->v_res))
+        return fail(BITDECODE_EINVAL, "tensor pointers must be 16-byte aligned");
+    const int64_t strides[8] = {a->q_stride_b, a->q_stride_h, a->kres_stride_b, a->kres_stride_t, a->kres_stride_h,
+                                a->vres_stride_b, a->vres_stride_t, a->vres_stride_h};
+    for (int64_t s : strides)
+        if (s % 8) return fail(BITDECODE_EINVAL, "q and residual strides must be multiples of 8 elements");
+
+    int nsplit = a->num_splits;
+    if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
+    if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, units_of(max_s, max_r), query_cus());
+    if (nsplit > 1) {
+        const size_t need = bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
+        if (!a->workspace || a->workspace_bytes < need)
+            return fail(BITDECODE_EWORKSPACE, "workspace of %zu bytes needed for %d splits, got %zu", need, nsplit,
+                        a->workspace ? a->workspace_bytes : size_t(0));
+        if (!aligned16(a->workspace)) return fail(BITDECODE_EINVAL, "workspace must be 16-byte aligned");
+    }
+
+    FwdParams P{};
+    P.q = static_cast<const uint16_t*>(a->q);
+    P.q_sb = a->q_stride_b; P.q_sh = a->q_stride_h;
+    P.k_pack = static_cast<const uint8_t*>(a->k_pack);
+    P.k_params = static_cast<const uint8_t*>(a->k_params);
+    P.v_pack = static_cast<const uint8_t*>(a->v_pack);
+    P.v_params = static_cast<const uint8_t*>(a->v_params);
+    P.kpack_bh = code_region_bytes(a->cache_tokens, a->bits);
+    P.vpack_bh = P.kpack_bh;
+    P.kparams_bh = k_param_region_bytes(a->cache_tokens, a->group_size);
+    P.vparams_bh = v_param_region_bytes(a->cache_tokens, a->group_size);
+    P.k_res = static_cast<const uint16_t*>(a->k_res);
+    P.v_res = static_cast<const uint16_t*>(a->v_res);
+    P.kres_sb = a->kres_stride_b; P.kres_st = a->kres_stride_t; P.kres_sh = a->kres_stride_h;
+    P.vres_sb = a->vres_stride_b; P.vres_st = a->vres_stride_t; P.vres_sh = a->vres_stride_h;
+    P.seqlens = a->seqlens_k; P.reslens = a->res_lens;
+    P.seqlen = a->seqlen_k; P.reslen = a->res_len;
+    P.out = static_cast<uint16_t*>(a->out);
+    P.out_sb = a->out_stride_b; P.out_sh = a->out_stride_h;
+    P.lse = a->softmax_lse;
+    P.b = a->b; P.h = a->h; P.hk = a->h_k; P.g = g; P.nsplit = nsplit;
+    P.scale = a->softmax_scale;
+    P.scale_log2 = a->softmax_scale * 1.4426950408889634f;   // decode_api.cpp:128-142
+    P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
+    if (nsplit > 1) {
+        P.o_part = static_cast<float*>(a->workspace);
+        P.lse_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
+    }
+    hipError_t e = launch_fwd(P, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));
+    return BITDECODE_OK;
+}
+
+}  // extern "C"

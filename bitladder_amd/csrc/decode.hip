@@ -1,0 +1,579 @@
+// Split-KV decode attention over [packed low-bit prefix || fp16 residual window] + LSE combine.
+//
+// Replaces compute_attn_1rowblock_splitkv and combine_attn_seqk_parallel of the reference
+// (csrc/bit_decode/src/flash_fwd_kernel.h:66-728, 1144-1327) with a wave64/MFMA design:
+//
+//  * A workgroup owns one (split, kv-head, batch); each of its waves streams whole work units of
+//    that split: a packed 128-token chunk (~17 KB at 4 bits) or a 32-token fp16 block (16 KB).
+//    All chunk data is fetched with 16-byte lane loads that form contiguous 1 KB wave rows.
+//  * Both products are computed transposed on v_mfma_f32_16x16x32_f16:
+//        S^T = K * Q^T   (A = K codes, row = token; B = Q, column = query head of the GQA group)
+//        O^T = V^T * P^T (A = V codes, row = channel; B = P^T)
+//    so the accumulator registers of the first product are, lane for lane, the B operand of the
+//    second one: P never leaves registers.
+//  * Codes are never multiplied out.  A dword of codes becomes four half2 registers holding
+//    (offset + code) through a mask and an exponent OR (dequantize.h:59-166 uses the same magic
+//    numbers); the per-channel K scale is folded into Q once per group, the per-token V scale is
+//    folded into P, and the offset/zero terms become one scalar bias per head:
+//        q.k_n   = sum_c (q_c*s_c)*(off + code) + sum_c q_c*z_c - sum_c (q_c*s_c)*off
+//        o_c     = sum_n (p_n*s_n)*(off + code) + sum_n p_n*z_n - sum_n (p_n*s_n)*off
+//  * q*scale and p*scale do not fit fp16 (11+11 significant bits), and their rounding error would
+//    multiply the large code*scale terms of outlier channels.  Each product is therefore kept as
+//    an exact pair hi + lo (lo = fma(a, b, -hi)).  The 16 MFMA columns hold the GQA group twice:
+//    columns 0-7 carry the hi parts of heads 0-7, columns 8-15 the lo parts, so both go through
+//    the same MFMA and are added afterwards with one row-rotate (lane ^ 8) per accumulator.
+//  * Online softmax in base 2 per head (softmax.h:250-310), running max shared by the four
+//    lanes of a head through two cross-lane exchanges, row sums kept per lane until the end.
+//  * The waves of a workgroup merge through LDS, splits merge in the combine kernel.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kernels.h"
+#include "layout.h"
+
+namespace bitdecode {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+
+constexpr int kNW = 8;            // waves per workgroup
+constexpr float kPShift = 2.0f;   // probabilities are kept as 2^kPShift * exp2(s - max): a V scale
+                                  // is at most 65504*2/3, so p*scale cannot overflow fp16
+constexpr int kLdsRowHalves = 136;
+
+__device__ __forceinline__ h2 pk_rtz(float a, float b) {
+    return __builtin_bit_cast(h2, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+
+// 16 bytes of fp16 (or bf16 converted to fp16; exact inside the fp16 normal range)
+template <bool BF16>
+__device__ __forceinline__ h8 cvt_h8(u4 raw) {
+    if constexpr (BF16) {
+        h8 r;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            h2 t = pk_rtz(__uint_as_float(raw[x] << 16), __uint_as_float(raw[x] & 0xffff0000u));
+            r[2 * x] = t[0];
+            r[2 * x + 1] = t[1];
+        }
+        return r;
+    } else {
+        return __builtin_bit_cast(h8, raw);
+    }
+}
+
+template <bool BF16>
+__device__ __forceinline__ h8 ld_h8(const void* p) {
+    return cvt_h8<BF16>(*reinterpret_cast<const u4*>(p));
+}
+
+__device__ __forceinline__ u4 ld_u4(const void* p) { return *reinterpret_cast<const u4*>(p); }
+
+__device__ __forceinline__ float dot8(h8 a, h8 b, float c) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        h2 a2 = {a[2 * x], a[2 * x + 1]};
+        h2 b2 = {b[2 * x], b[2 * x + 1]};
+        c = __builtin_amdgcn_fdot2(a2, b2, c, false);
+    }
+    return c;
+}
+
+// 8 four-bit codes -> (1024+c0, 1024+c4, 64+c1, 64+c5, 1024+c2, 1024+c6, 64+c3, 64+c7)
+__device__ __forceinline__ h8 dq4(uint32_t w) {
+    u4 r;
+    r[0] = (w & 0x000f000fu) | 0x64006400u;
+    r[1] = (w & 0x00f000f0u) | 0x54005400u;
+    const uint32_t w8 = w >> 8;
+    r[2] = (w8 & 0x000f000fu) | 0x64006400u;
+    r[3] = (w8 & 0x00f000f0u) | 0x54005400u;
+    return __builtin_bit_cast(h8, r);
+}
+// 16 two-bit codes -> two k-steps; offsets per element (1024,1024,256,256,64,64,16,16)
+__device__ __forceinline__ void dq2(uint32_t w, h8& a0, h8& a1) {
+    u4 r;
+    r[0] = (w & 0x00030003u) | 0x64006400u;
+    r[1] = (w & 0x000c000cu) | 0x5c005c00u;
+    r[2] = (w & 0x00300030u) | 0x54005400u;
+    r[3] = (w & 0x00c000c0u) | 0x4c004c00u;
+    a0 = __builtin_bit_cast(h8, r);
+    const uint32_t w8 = w >> 8;
+    r[0] = (w8 & 0x00030003u) | 0x64006400u;
+    r[1] = (w8 & 0x000c000cu) | 0x5c005c00u;
+    r[2] = (w8 & 0x00300030u) | 0x54005400u;
+    r[3] = (w8 & 0x00c000c0u) | 0x4c004c00u;
+    a1 = __builtin_bit_cast(h8, r);
+}
+
+template <int BITS>
+__device__ __forceinline__ h8 code_offsets() {
+    if constexpr (BITS == 4) {
+        return h8{1024, 1024, 64, 64, 1024, 1024, 64, 64};
+    } else {
+        return h8{1024, 1024, 256, 256, 64, 64, 16, 16};
+    }
+}
+
+__device__ __forceinline__ f4 mfma32(h8 a, h8 b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+}
+
+// value held by the partner column (lane ^ 8 inside each row of 16 lanes): DPP row_ror:8
+__device__ __forceinline__ float partner(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
+}
+// exact product a*b as hi + lo in fp16; returns the part this column carries
+__device__ __forceinline__ h8 split_mul(h8 a, h8 b, bool lo_part) {
+    const h8 hi = a * b;
+    const h8 lo = __builtin_elementwise_fma(a, b, -hi);
+    return lo_part ? lo : hi;
+}
+
+// sum / max over the four lanes that share a column (lane, lane^16, lane^32, lane^48)
+__device__ __forceinline__ float colsum(float x) {
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
+}
+__device__ __forceinline__ float colmax(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16));
+    x = fmaxf(x, __shfl_xor(x, 32));
+    return x;
+}
+
+template <int NCG>
+struct WaveState {
+    float m;          // running max of the base-2 scores of this lane's head
+    float l;          // this lane's share of sum p
+    float bv[NCG];    // this lane's share of the V bias per channel group
+    f4 o[8];          // O^T tiles: lane (head, q) holds channels 16*ct + 4*q + r
+};
+
+// Online-softmax step over N scores; returns p = 2^kPShift * exp2(s - max) in place.
+template <int N, int NCG>
+__device__ __forceinline__ void softmax_step(float (&s)[N], WaveState<NCG>& st) {
+    float mx = s[0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) mx = fmaxf(mx, s[i]);
+    mx = colmax(mx);
+    const float m_new = fmaxf(st.m, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
+#pragma unroll
+    for (int i = 0; i < N; ++i) s[i] = __builtin_amdgcn_exp2f(s[i] - m_use + kPShift);
+    st.l *= alpha;
+#pragma unroll
+    for (int c = 0; c < NCG; ++c) st.bv[c] *= alpha;
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) st.o[ct] *= alpha;
+    st.m = m_new;
+}
+
+// ---------------------------------------------------------------------------------------------
+// one packed 128-token chunk
+// ---------------------------------------------------------------------------------------------
+template <int BITS, int GS, bool BF16>
+__device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int ci, int lane,
+                                             const h8 (&qB)[4], bool lo_part,
+                                             WaveState<kHeadDim / GS>& st) {
+    constexpr int NG = kChunk / GS;
+    constexpr int NCG = kHeadDim / GS;
+    constexpr int TPG = GS / 16;      // 16-token tiles per K group
+    constexpr int CTPG = GS / 16;     // 16-channel tiles per V channel group
+    const int kg = lane >> 4;
+    const h8 off = code_offsets<BITS>();
+    const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
+
+    const uint8_t* kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
+    const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
+    const uint8_t* vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
+    const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
+
+    // ---- S^T = K Q^T for the 8 tiles of the chunk
+    float s[32];
+#pragma unroll
+    for (int grp = 0; grp < NG; ++grp) {
+        h8 qp[4];
+        float kap = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const h8 sc = ld_h8<BF16>(kp + grp * kKParamGroupBytes + (32 * j + 8 * kg) * 2);
+            const h8 zr = ld_h8<BF16>(kp + grp * kKParamGroupBytes + 256 + (32 * j + 8 * kg) * 2);
+            qp[j] = split_mul(qB[j], sc, lo_part);
+            if (!lo_part) kap = dot8(qB[j], zr, kap);
+            kap = -dot8(qp[j], off, -kap);
+        }
+        kap = colsum(kap) * P.scale_log2;
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int tt = 0; tt < TPG; ++tt) {
+                const int t = grp * TPG + tt;
+                const u4 w = ld_u4(kc + t * 1024 + lane * 16);
+                f4 acc = {0, 0, 0, 0};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc = mfma32(dq4(w[j]), qp[j], acc);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float sp = acc[r] * P.scale_log2 + kap;
+                    s[4 * t + r] = sp + partner(sp);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int pp = 0; pp < TPG / 2; ++pp) {
+                const int tp = grp * (TPG / 2) + pp;
+                const u4 w = ld_u4(kc + tp * 1024 + lane * 16);
+#pragma unroll
+                for (int tin = 0; tin < 2; ++tin) {
+                    f4 acc = {0, 0, 0, 0};
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+                        h8 a0, a1;
+                        dq2(w[2 * tin + jj], a0, a1);
+                        acc = mfma32(a0, qp[2 * jj], acc);
+                        acc = mfma32(a1, qp[2 * jj + 1], acc);
+                    }
+                    const int t = 2 * tp + tin;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float sp = acc[r] * P.scale_log2 + kap;
+                        s[4 * t + r] = sp + partner(sp);
+                    }
+                }
+            }
+        }
+    }
+
+    softmax_step<32, NCG>(s, st);
+
+    // ---- O^T += V^T P^T, 32 tokens (one k-step) at a time
+    h8 p16[4];
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            // element i = 4*T + r  <->  tile 2*sb + T, accumulator register r
+            const int i0 = 2 * x;
+            const int t0 = 2 * sb + i0 / 4, r0 = i0 % 4;
+            h2 t = pk_rtz(s[4 * t0 + r0], s[4 * t0 + r0 + 1]);
+            p16[sb][2 * x] = t[0];
+            p16[sb][2 * x + 1] = t[1];
+        }
+        st.l = dot8(p16[sb], ones, st.l);
+    }
+
+    if constexpr (BITS == 4) {
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb) {
+            const u4 w0 = ld_u4(vc + sb * 2048 + lane * 16);
+            const u4 w1 = ld_u4(vc + sb * 2048 + 1024 + lane * 16);
+#pragma unroll
+            for (int cg = 0; cg < NCG; ++cg) {
+                const h8 vs = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + kg * 16);
+                const h8 vz = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + 64 + kg * 16);
+                const h8 pp = split_mul(p16[sb], vs, lo_part);
+                if (!lo_part) st.bv[cg] = dot8(p16[sb], vz, st.bv[cg]);
+                st.bv[cg] = -dot8(pp, off, -st.bv[cg]);
+#pragma unroll
+                for (int x = 0; x < CTPG; ++x) {
+                    const int ct = cg * CTPG + x;
+                    const uint32_t w = ct < 4 ? w0[ct & 3] : w1[ct & 3];
+                    st.o[ct] = mfma32(dq4(w), pp, st.o[ct]);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int sb2 = 0; sb2 < 2; ++sb2) {
+            const u4 w0 = ld_u4(vc + sb2 * 2048 + lane * 16);
+            const u4 w1 = ld_u4(vc + sb2 * 2048 + 1024 + lane * 16);
+#pragma unroll
+            for (int cg = 0; cg < NCG; ++cg) {
+                h8 pp[2];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    const int sb = 2 * sb2 + ks;
+                    const h8 vs = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + kg * 16);
+                    const h8 vz = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + 64 + kg * 16);
+                    pp[ks] = split_mul(p16[sb], vs, lo_part);
+                    if (!lo_part) st.bv[cg] = dot8(p16[sb], vz, st.bv[cg]);
+                    st.bv[cg] = -dot8(pp[ks], off, -st.bv[cg]);
+                }
+#pragma unroll
+                for (int x = 0; x < CTPG; ++x) {
+                    const int ct = cg * CTPG + x;
+                    const uint32_t w = ct < 4 ? w0[ct & 3] : w1[ct & 3];
+                    h8 a0, a1;
+                    dq2(w, a0, a1);
+                    st.o[ct] = mfma32(a0, pp[0], st.o[ct]);
+                    st.o[ct] = mfma32(a1, pp[1], st.o[ct]);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// one 32-token block of the fp16 residual window (tokens n0 .. n0+31, valid below R)
+// ---------------------------------------------------------------------------------------------
+template <bool BF16, int NCG>
+__device__ __forceinline__ void fp16_block(const FwdParams& P, int bi, int hk, int n0, int R, int lane,
+                                           const h8 (&qB)[4], bool lo_part, WaveState<NCG>& st,
+                                           uint16_t* lds) {
+    const int col = lane & 15, kg = lane >> 4;
+    const h8 zero8 = h8{0, 0, 0, 0, 0, 0, 0, 0};
+    const uint16_t* kr = P.k_res + bi * P.kres_sb + hk * P.kres_sh;
+    const uint16_t* vr = P.v_res + bi * P.vres_sb + hk * P.vres_sh;
+    const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
+
+    float s[8];
+#pragma unroll
+    for (int T = 0; T < 2; ++T) {
+        const int tok = n0 + 16 * T + col;
+        f4 acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            h8 a = h8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (tok < R) a = ld_h8<BF16>(kr + static_cast<int64_t>(tok) * P.kres_st + 32 * j + 8 * kg);
+            acc = mfma32(a, lo_part ? zero8 : qB[j], acc);   // fp16 operands are exact: no lo part
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int tk = n0 + 16 * T + 4 * kg + r;
+            const float sp = acc[r] * P.scale_log2;
+            const float tot = sp + partner(sp);     // outside the select: every lane must execute the DPP
+            s[4 * T + r] = tk < R ? tot : -INFINITY;
+        }
+    }
+    softmax_step<8, NCG>(s, st);
+    h8 p16;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        h2 t = pk_rtz(s[2 * x], s[2 * x + 1]);
+        p16[2 * x] = t[0];
+        p16[2 * x + 1] = t[1];
+    }
+    st.l = dot8(p16, ones, st.l);
+
+    // V tile (16 tokens x 128 channels) goes through this wave's LDS slab to be read back
+    // token-contiguous per channel (the MFMA A operand wants 4 tokens of one channel per lane).
+#pragma unroll
+    for (int T = 0; T < 2; ++T) {
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int tl = 4 * x + kg;
+            const int tok = n0 + 16 * T + tl;
+            u4 d = {0, 0, 0, 0};
+            if (tok < R) d = ld_u4(vr + static_cast<int64_t>(tok) * P.vres_st + col * 8);
+            *reinterpret_cast<u4*>(&lds[tl * kLdsRowHalves + col * 8]) = d;
+        }
+        __builtin_amdgcn_wave_barrier();
+        h4 pb = {p16[4 * T], p16[4 * T + 1], p16[4 * T + 2], p16[4 * T + 3]};
+        if (lo_part) pb = h4{0, 0, 0, 0};
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+            uint16_t e[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) e[i] = lds[(4 * kg + i) * kLdsRowHalves + 16 * ct + col];
+            h4 a;
+            if constexpr (BF16) {
+                h2 t0 = pk_rtz(__uint_as_float(static_cast<uint32_t>(e[0]) << 16),
+                               __uint_as_float(static_cast<uint32_t>(e[1]) << 16));
+                h2 t1 = pk_rtz(__uint_as_float(static_cast<uint32_t>(e[2]) << 16),
+                               __uint_as_float(static_cast<uint32_t>(e[3]) << 16));
+                a = h4{t0[0], t0[1], t1[0], t1[1]};
+            } else {
+                a = h4{__builtin_bit_cast(_Float16, e[0]), __builtin_bit_cast(_Float16, e[1]),
+                       __builtin_bit_cast(_Float16, e[2]), __builtin_bit_cast(_Float16, e[3])};
+            }
+            st.o[ct] = mfma16(a, pb, st.o[ct]);
+        }
+    }
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint16_t to_out(float f) {
+    if constexpr (BF16) {
+        uint32_t u = __float_as_uint(f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return static_cast<uint16_t>(u >> 16);
+    } else {
+        return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// split-KV kernel: grid (num_splits, h_k, b), kNW waves
+// ---------------------------------------------------------------------------------------------
+template <int BITS, int GS, bool BF16>
+__global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
+    constexpr int NCG = kHeadDim / GS;
+    constexpr int kSlabHalves = 16 * kLdsRowHalves;
+    constexpr int kMergeFloats = kNW * kMaxGroupHeads * kHeadDim;
+    constexpr int kLdsBytes = (kMergeFloats * 4 > kNW * kSlabHalves * 2) ? kMergeFloats * 4 : kNW * kSlabHalves * 2;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kLdsBytes];
+    __shared__ float sM[kNW][kMaxGroupHeads], sL[kNW][kMaxGroupHeads];
+
+    const int split = blockIdx.x, hk = blockIdx.y, bi = blockIdx.z;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 15, kg = lane >> 4;
+    const int head = col & 7;          // query head inside the GQA group
+    const bool lo_part = col >= 8;     // columns 8-15 carry the lo halves of the split products
+    const int g = P.g;
+    const int64_t bh = static_cast<int64_t>(bi) * P.hk + hk;
+
+    const int S = P.seqlens ? P.seqlens[bi] : P.seqlen;
+    const int R = P.reslens ? P.reslens[bi] : P.reslen;
+    const int nP = S / kChunk, nR = (R + 31) / 32, U = nP + nR;
+    const int ups = (U + P.nsplit - 1) / P.nsplit;
+    const int u0 = split * ups;
+    const int u1 = min(U, u0 + ups);
+
+    h8 qB[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        qB[j] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (head < g) qB[j] = ld_h8<BF16>(P.q + bi * P.q_sb + (hk * g + head) * P.q_sh + 32 * j + 8 * kg);
+    }
+
+    WaveState<NCG> st;
+    st.m = -INFINITY;
+    st.l = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCG; ++c) st.bv[c] = 0.0f;
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) st.o[ct] = f4{0, 0, 0, 0};
+
+    uint16_t* slab = reinterpret_cast<uint16_t*>(lds_raw) + wave * kSlabHalves;
+    for (int u = u0 + wave; u < u1; u += kNW) {
+        if (u < nP) {
+            packed_chunk<BITS, GS, BF16>(P, bh, u, lane, qB, lo_part, st);
+        } else {
+            fp16_block<BF16, NCG>(P, bi, hk, (u - nP) * 32, R, lane, qB, lo_part, st, slab);
+        }
+    }
+
+    // ---- merge the waves of this workgroup through LDS
+    st.l = colsum(st.l);
+#pragma unroll
+    for (int c = 0; c < NCG; ++c) st.bv[c] = colsum(st.bv[c]);
+    __syncthreads();   // slabs are dead from here on
+    float* sO = reinterpret_cast<float*>(lds_raw);
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) {
+        const float bias = st.bv[ct / (GS / 16)];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = st.o[ct][r] + bias;
+            st.o[ct][r] = v + partner(v);      // hi + lo
+        }
+    }
+    if (col < g) {
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+            *reinterpret_cast<f4*>(&sO[(wave * kMaxGroupHeads + col) * kHeadDim + 16 * ct + 4 * kg]) = st.o[ct];
+        }
+        if (kg == 0) {
+            sM[wave][col] = st.m;
+            sL[wave][col] = st.l;
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < g * kHeadDim; idx += kNW * 64) {
+        const int hh = idx >> 7, c = idx & 127;
+        float M = sM[0][hh];
+#pragma unroll
+        for (int w = 1; w < kNW; ++w) M = fmaxf(M, sM[w][hh]);
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kNW; ++w) {
+            const float a = __builtin_amdgcn_exp2f(sM[w][hh] - Mu);
+            L += a * sL[w][hh];
+            O += a * sO[(w * kMaxGroupHeads + hh) * kHeadDim + c];
+        }
+        const bool empty = !(L > 0.0f);
+        const float o = empty ? 0.0f : O / L;
+        // natural-log LSE of this split (softmax.h:303); -inf marks an empty split
+        const float lse = empty ? -INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+        const int hq = hk * g + hh;
+        if (P.nsplit == 1) {
+            P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(o);
+            if (c == 0 && P.lse) P.lse[bi * P.h + hq] = empty ? INFINITY : lse;
+        } else {
+            const int64_t row = (static_cast<int64_t>(split) * P.b + bi) * P.h + hq;
+            P.o_part[row * kHeadDim + c] = o;
+            if (c == 0) P.lse_part[row] = lse;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// combine kernel: grid (b*h), 128 threads; follows flash_fwd_kernel.h:1217-1248, 1280-1298
+// ---------------------------------------------------------------------------------------------
+template <bool BF16>
+__global__ __launch_bounds__(128) void combine_kernel(FwdParams P) {
+    const int row = blockIdx.x;           // bi * h + hq
+    const int bi = row / P.h, hq = row % P.h;
+    const int c = threadIdx.x;
+    const int64_t stride = static_cast<int64_t>(P.b) * P.h;
+    float M = -INFINITY;
+    for (int s = 0; s < P.nsplit; ++s) M = fmaxf(M, P.lse_part[s * stride + row]);
+    const float Mu = (M == -INFINITY) ? 0.0f : M;
+    float sum = 0.0f;
+    for (int s = 0; s < P.nsplit; ++s) sum += __expf(P.lse_part[s * stride + row] - Mu);
+    const float L = (sum == 0.0f || sum != sum) ? INFINITY : __logf(sum) + Mu;
+    float o = 0.0f;
+    for (int s = 0; s < P.nsplit; ++s) {
+        const float w = __expf(P.lse_part[s * stride + row] - L);
+        o += w * P.o_part[(s * stride + row) * kHeadDim + c];
+    }
+    P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(o);
+    if (c == 0 && P.lse) P.lse[row] = L;
+}
+
+template <int BITS, int GS>
+hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
+    dim3 grid(P.nsplit, P.hk, P.b);
+    if (P.bf16) {
+        hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, true>), grid, dim3(kNW * 64), 0, stream, P);
+    } else {
+        hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, false>), grid, dim3(kNW * 64), 0, stream, P);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (P.nsplit > 1) {
+        if (P.bf16) {
+            hipLaunchKernelGGL((combine_kernel<true>), dim3(P.b * P.h), dim3(128), 0, stream, P);
+        } else {
+            hipLaunchKernelGGL((combine_kernel<false>), dim3(P.b * P.h), dim3(128), 0, stream, P);
+        }
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+}  // namespace
+
+hipError_t launch_fwd(const FwdParams& P, hipStream_t stream) {
+    switch (P.bits * 1000 + P.gs) {
+        case 4128: return launch_fwd_t<4, 128>(P, stream);
+        case 4064: return launch_fwd_t<4, 64>(P, stream);
+        case 4032: return launch_fwd_t<4, 32>(P, stream);
+        case 2128: return launch_fwd_t<2, 128>(P, stream);
+        case 2064: return launch_fwd_t<2, 64>(P, stream);
+        case 2032: return launch_fwd_t<2, 32>(P, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace bitdecode

@@ -1,0 +1,50 @@
+// Internal launch interface between the C ABI (api.hip) and the kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bitdecode {
+
+struct QpackParams {
+    const uint16_t* k;
+    const uint16_t* v;
+    int64_t k_sb, k_st, k_sh, v_sb, v_st, v_sh;      // element strides
+    uint8_t* k_pack;
+    uint8_t* k_params;
+    uint8_t* v_pack;
+    uint8_t* v_params;
+    int64_t kpack_bh, kparams_bh, vpack_bh, vparams_bh;  // bytes per (batch, kv-head) region
+    int b, n_tokens, hk;
+    int dst_offset;
+    const int* dst_offsets;
+    int bits, gs, bf16;
+};
+
+struct FwdParams {
+    const uint16_t* q;
+    int64_t q_sb, q_sh;
+    const uint8_t* k_pack;
+    const uint8_t* k_params;
+    const uint8_t* v_pack;
+    const uint8_t* v_params;
+    int64_t kpack_bh, kparams_bh, vpack_bh, vparams_bh;
+    const uint16_t* k_res;
+    const uint16_t* v_res;
+    int64_t kres_sb, kres_st, kres_sh, vres_sb, vres_st, vres_sh;
+    const int* seqlens;
+    const int* reslens;
+    int seqlen, reslen;
+    float* o_part;      // [split][b][h][128] normalised partial outputs
+    float* lse_part;    // [split][b][h] natural-log LSE of each split
+    uint16_t* out;
+    int64_t out_sb, out_sh;
+    float* lse;         // optional [b][h]
+    int b, h, hk, g, nsplit;
+    float scale, scale_log2;
+    int bits, gs, bf16;
+};
+
+hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);
+hipError_t launch_fwd(const FwdParams& p, hipStream_t stream);
+
+}  // namespace bitdecode

@@ -1,0 +1,56 @@
+// Physical layout of the packed KV cache for gfx950 (wave64, 16-byte lane loads, MFMA 16x16x32).
+//
+// The caller allocates the four tensors with the reference's shapes
+//   k_pack   (b, S/pn, h_k, 128) u16      k_params (b, S/gs, h_k, 128) f32 (= 2 x fp16)
+//   v_pack   (b, S,    h_k, 128/pn) u16   v_params (b, 128/gs, h_k, S) f32 (= 2 x fp16)
+// (pn = 16/bits; reference: evaluation/test.py:76-83).  Only the byte budget of those shapes is
+// kept; the arrangement of bytes inside is private to this library's pack and decode kernels
+// and is described here.  S below is the capacity in tokens implied by the tensor shape.
+//
+// Every tensor is split into one contiguous region per (batch, kv-head), region index
+// b * h_k + h, and every region into 128-token chunks, so a decode wave streams one chunk of
+// one head as a run of fully coalesced 1 KB wave loads (64 lanes x 16 B).
+//
+// MFMA view used by the decode kernel (v_mfma_f32_16x16x32_f16, lane = col + 16*kg):
+//   QK^T is computed transposed, S^T = K * Q^T: A operand = K codes, row = token,
+//        8 k-values per lane = 8 channels;  B operand = Q, column = query head.
+//   PV is computed transposed, O^T = V^T * P^T: A operand = V codes, row = channel,
+//        8 k-values per lane = 8 tokens;  B operand = P^T straight out of the QK^T
+//        accumulator registers (no LDS round trip), which fixes the token order below.
+//
+// K codes, 4-bit: chunk = 8 tiles of 16 tokens, tile = 1 KB = 64 lanes x 4 dwords.
+//   lane l = m + 16*kg holds token 16*t + m; dword j, element i (0..7) is channel 32*j + 8*kg + i;
+//   element i sits in nibble p = i/2 + 4*(i%2) (so that two masks and one shift unpack a dword
+//   into four half2 registers).
+// K codes, 2-bit: chunk = 4 tile pairs, pair = 1 KB = 64 lanes x 4 dwords; dword dd = 2*tin + jj
+//   holds token 16*(2*tp + tin) + m, k-steps j = 2*jj and 2*jj+1: element e = 8*(j%2) + i sits in
+//   field f = e/2 + 8*(e%2), channel 32*j + 8*kg + i.
+// V codes, 4-bit: chunk = 4 sub-blocks of 32 tokens, sub-block = 2 halves x 1 KB; half hf,
+//   lane l = c + 16*kg, dword x: channel 16*(4*hf + x) + c; element i is token
+//   32*sb + 16*(i/4) + 4*kg + i%4, nibble p = i/2 + 4*(i%2).
+// V codes, 2-bit: chunk = 2 sub-blocks of 64 tokens, same halves/lanes/dwords; element
+//   e = 8*ks + i is token 64*sb2 + 32*ks + 16*(i/4) + 4*kg + i%4, field f = e/2 + 8*(e%2).
+// K params: per group of gs tokens 512 B: scale[128] then zero[128], natural channel order.
+// V params: per chunk 4 sub-blocks x ncg channel groups x 128 B: scale[q][i] (64 B) then
+//   zero[q][i] (64 B), q = 0..3, i = 0..7, token 32*sb + 16*(i/4) + 4*q + i%4.
+#pragma once
+#include <stdint.h>
+
+namespace bitdecode {
+
+constexpr int kHeadDim = 128;
+constexpr int kChunk = 128;               // tokens per chunk (pack granularity)
+constexpr int kMaxGroupHeads = 8;         // query heads per kv head handled by one MFMA tile
+
+// bytes of K (or V) codes per chunk
+constexpr int chunk_code_bytes(int bits) { return kChunk * kHeadDim * bits / 8; }
+// bytes of K params per token group / of V params per chunk
+constexpr int kKParamGroupBytes = 4 * kHeadDim;
+constexpr int v_param_chunk_bytes(int gs) { return kChunk * (kHeadDim / gs) * 4; }
+
+// per-(batch, kv-head) region sizes in bytes for a cache with capacity S tokens
+constexpr int64_t code_region_bytes(int64_t S, int bits) { return S * kHeadDim * bits / 8; }
+constexpr int64_t k_param_region_bytes(int64_t S, int gs) { return (S / gs) * kKParamGroupBytes; }
+constexpr int64_t v_param_region_bytes(int64_t S, int gs) { return S * (kHeadDim / gs) * 4; }
+
+}  // namespace bitdecode

@@ -1,0 +1,307 @@
+"""Python entry points of the low-bit KV-cache decode path, drop-in for the reference's
+`bit_decode/bit_decode_interface.py`: same names, positional order, defaults, tensor shapes and
+dtypes.  Host code is PyTorch (device memory, streams); all device work goes through the C ABI
+of libbitdecode.so (hand-written HIP for gfx950).  Keyword-only arguments are extensions.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Union
+
+import torch
+
+from . import _lib
+
+_PACK_DTYPES = (torch.uint16, torch.int16)
+CHUNK = 128
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return _lib.FP16
+    if t.dtype == torch.bfloat16:
+        return _lib.BF16
+    # decode_api.cpp:531-533: "only support fp16 and bf16 data type"
+    raise RuntimeError("bit_decode only supports fp16 and bf16 data type")
+
+
+def _check_quant(quant_mode: str, group_size: int, num_bits: int) -> None:
+    if quant_mode != "k-channel":
+        # the reference's "k-tensor" instantiations are commented out (decode_api.cpp:195-203)
+        raise NotImplementedError(f"quant_mode {quant_mode!r} is not supported (only 'k-channel')")
+    if num_bits not in (2, 4):
+        raise ValueError(f"num_bits must be 2 or 4, got {num_bits}")
+    if group_size not in (32, 64, 128):
+        raise ValueError(f"group_size must be 32, 64 or 128, got {group_size}")
+
+
+def _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device):
+    """Validates the caller-allocated packed tensors (evaluation/test.py:74-83) and returns
+    (batch, capacity_tokens, h_k)."""
+    pn = 16 // num_bits
+    if v_pack.dim() != 4 or k_pack.dim() != 4 or k_params.dim() != 4 or v_params.dim() != 4:
+        raise RuntimeError("k_pack, k_params, v_pack, v_params must be 4-dimensional")
+    b, S, h_k, dp = v_pack.shape
+    d = dp * pn
+    if d != 128:
+        raise RuntimeError(f"head dimension {d} is not supported (only 128)")
+    if S % CHUNK:
+        raise RuntimeError(f"packed cache capacity {S} must be a multiple of {CHUNK} tokens")
+    want = {
+        "k_pack": (b, S // pn, h_k, d), "k_params": (b, S // group_size, h_k, d),
+        "v_pack": (b, S, h_k, d // pn), "v_params": (b, d // group_size, h_k, S),
+    }
+    for name, t in (("k_pack", k_pack), ("k_params", k_params), ("v_pack", v_pack), ("v_params", v_params)):
+        if tuple(t.shape) != want[name]:
+            raise RuntimeError(f"{name} must have shape {want[name]}, got {tuple(t.shape)}")
+        if t.device != device:
+            raise RuntimeError(f"{name} must be on {device}")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    for name, t in (("k_pack", k_pack), ("v_pack", v_pack)):
+        if t.dtype not in _PACK_DTYPES:
+            raise RuntimeError(f"{name} must have dtype torch.uint16")
+    for name, t in (("k_params", k_params), ("v_params", v_params)):
+        if t.dtype != torch.float32:
+            raise RuntimeError(f"{name} must have dtype torch.float32 (each element holds two 16-bit values)")
+    return b, S, h_k
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _i32_dev(x, b, device, name):
+    if not isinstance(x, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if x.dtype != torch.int32 or x.device != device or not x.is_contiguous() or x.numel() != b:
+        raise RuntimeError(f"{name} must be a contiguous int32 tensor of {b} elements on {device}")
+    return x
+
+
+def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torch.Tensor,
+                     v_cache: torch.Tensor, v_pack: torch.Tensor, v_params: torch.Tensor,
+                     opt_block_table: Optional[torch.Tensor] = None,
+                     cu_seqlens_k: torch.Tensor = None,
+                     seqlen_k: int = 0,
+                     quant_mode: str = "k-channel",
+                     group_size: int = 128,
+                     num_bits: int = 4,
+                     *,
+                     dst_offset: int = 0,
+                     dst_offsets: Optional[torch.Tensor] = None) -> None:
+    """Quantize-pack `k_cache`/`v_cache` [b, n, h_k, 128] into the caller-allocated packed cache
+    (reference: bit_decode_interface.py:10-41).  K is quantized per channel, V per token.
+
+    As in the reference `seqlen_k` is ignored in favour of `k_cache.shape[1]` and `cu_seqlens_k`
+    is only validated (decode_api.cpp:537-541, 585).  Extensions: `dst_offset` (int) or
+    `dst_offsets` (int32 [b] device tensor) give the token position, a multiple of 128, at which
+    the n new tokens are written, so a full fp16 residual block can be appended to the cache.
+    """
+    _check_quant(quant_mode, group_size, num_bits)
+    if opt_block_table is not None:
+        raise NotImplementedError("paged KV cache (opt_block_table) is not supported")
+    if k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
+        raise RuntimeError("k_cache and v_cache must both be [batch, seqlen, nheads_k, head_dim]")
+    if not k_cache.is_cuda:
+        raise RuntimeError("k_cache must be on a GPU device")
+    if v_cache.dtype != k_cache.dtype or v_cache.device != k_cache.device:
+        raise RuntimeError("k_cache and v_cache must have the same dtype and device")
+    dtype = _dtype_code(k_cache)
+    device = k_cache.device
+    b, n, h_k, d = k_cache.shape
+    cb, S, ch_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device)
+    if (cb, ch_k) != (b, h_k) or d != 128:
+        raise RuntimeError("packed cache shape does not match k_cache")
+    if cu_seqlens_k is not None:
+        if cu_seqlens_k.dtype != torch.int32:
+            raise RuntimeError("cu_seqlens_k must have dtype int32")
+        if not cu_seqlens_k.is_contiguous():
+            raise RuntimeError("cu_seqlens_k must be contiguous")
+    if k_cache.stride(3) != 1 or v_cache.stride(3) != 1:
+        raise RuntimeError("Input tensor must have contiguous last dimension")
+    if n % CHUNK:
+        raise RuntimeError(f"number of tokens to pack ({n}) must be a multiple of {CHUNK}; "
+                           "keep the remainder in the fp16 residual window")
+
+    a = _lib.QpackArgs()
+    a.k, a.v = k_cache.data_ptr(), v_cache.data_ptr()
+    a.k_stride_b, a.k_stride_t, a.k_stride_h = k_cache.stride(0), k_cache.stride(1), k_cache.stride(2)
+    a.v_stride_b, a.v_stride_t, a.v_stride_h = v_cache.stride(0), v_cache.stride(1), v_cache.stride(2)
+    a.k_pack, a.k_params = k_pack.data_ptr(), k_params.data_ptr()
+    a.v_pack, a.v_params = v_pack.data_ptr(), v_params.data_ptr()
+    a.b, a.n_tokens, a.h_k, a.d = b, n, h_k, d
+    a.cache_tokens = S
+    a.dst_offset = int(dst_offset)
+    a.dst_offsets = None if dst_offsets is None else _i32_dev(dst_offsets, b, device, "dst_offsets").data_ptr()
+    a.bits, a.group_size, a.dtype = num_bits, group_size, dtype
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().bitdecode_qpack(ctypes.byref(a), _stream_ptr(device)))
+
+
+class DecodePlan:
+    """A validated decode call with its argument block and workspace held ready, so that
+    `run()` is one C-ABI call with no allocation (serving loops, HIP-graph capture).
+    Built by `plan_fwd_kvcache_int`; the tensors it was built from must stay alive and in place.
+    """
+
+    def __init__(self, args: "_lib.FwdArgs", out: torch.Tensor, lse: Optional[torch.Tensor],
+                 keep: tuple, device: torch.device):
+        self.args = args
+        self.out = out
+        self.lse = lse
+        self._keep = keep
+        self.device = device
+        self.num_splits = args.num_splits
+        self._fn = _lib.lib().bitdecode_fwd
+        self._ref = ctypes.byref(args)
+
+    def run(self, stream: Optional[int] = None) -> torch.Tensor:
+        rc = self._fn(self._ref, _stream_ptr(self.device) if stream is None else stream)
+        if rc:
+            _lib.check(rc)
+        return self.out
+
+
+def plan_fwd_kvcache_int(q: torch.Tensor,
+                         k_pack: torch.Tensor, k_params: torch.Tensor,
+                         v_pack: torch.Tensor, v_params: torch.Tensor,
+                         opt_block_table: Optional[torch.Tensor] = None,
+                         softmax_scale: float = 1.0,
+                         quant_mode: str = "k-channel",
+                         group_size: int = 128,
+                         num_bits: int = 4,
+                         *,
+                         seqlen_k: Optional[int] = None,
+                         seqlens_k: Optional[torch.Tensor] = None,
+                         max_seqlen_k: Optional[int] = None,
+                         k_residual: Optional[torch.Tensor] = None,
+                         v_residual: Optional[torch.Tensor] = None,
+                         residual_len: Union[int, torch.Tensor, None] = None,
+                         max_residual_len: Optional[int] = None,
+                         num_splits: int = 0,
+                         out: Optional[torch.Tensor] = None,
+                         return_lse: bool = False) -> DecodePlan:
+    """Validates a decode call and returns a `DecodePlan`; see `fwd_kvcache_int`."""
+    _check_quant(quant_mode, group_size, num_bits)
+    if opt_block_table is not None:
+        raise NotImplementedError("paged KV cache (opt_block_table) is not supported")
+    if q.dim() != 4 or q.shape[1] != 1:
+        raise RuntimeError("q must be [batch, 1, nheads, head_dim] (one query token per sequence)")
+    if not q.is_cuda:
+        raise RuntimeError("q must be on a GPU device")
+    dtype = _dtype_code(q)
+    device = q.device
+    b, _, h, d = q.shape
+    cb, S, h_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device)
+    if cb != b:
+        raise RuntimeError(f"batch size of q ({b}) and of the packed cache ({cb}) differ")
+    if d != 128:
+        raise RuntimeError("head dimension must be 128")
+    if h % h_k:
+        raise RuntimeError("Number of heads in key/value must divide number of heads in query")
+    if q.stride(3) != 1:
+        raise RuntimeError("Input tensor must have contiguous last dimension")
+
+    a = _lib.FwdArgs()
+    keep = [q, k_pack, k_params, v_pack, v_params]
+    a.q, a.q_stride_b, a.q_stride_h = q.data_ptr(), q.stride(0), q.stride(2)
+    a.k_pack, a.k_params = k_pack.data_ptr(), k_params.data_ptr()
+    a.v_pack, a.v_params = v_pack.data_ptr(), v_params.data_ptr()
+    a.cache_tokens = S
+    a.seqlen_k = S if seqlen_k is None else int(seqlen_k)
+    a.max_seqlen_k = a.seqlen_k
+    if seqlens_k is not None:
+        keep.append(_i32_dev(seqlens_k, b, device, "seqlens_k"))
+        a.seqlens_k = seqlens_k.data_ptr()
+        a.max_seqlen_k = S if max_seqlen_k is None else int(max_seqlen_k)
+    if (k_residual is None) != (v_residual is None):
+        raise RuntimeError("k_residual and v_residual must be given together")
+    if k_residual is not None:
+        for name, t in (("k_residual", k_residual), ("v_residual", v_residual)):
+            if t.dim() != 4 or t.shape[0] != b or t.shape[2] != h_k or t.shape[3] != d:
+                raise RuntimeError(f"{name} must be [batch, R, nheads_k, head_dim]")
+            if t.dtype != q.dtype or t.device != device:
+                raise RuntimeError(f"{name} must have the dtype and device of q")
+            if t.stride(3) != 1:
+                raise RuntimeError(f"{name} must have contiguous last dimension")
+        if v_residual.shape[1] != k_residual.shape[1]:
+            raise RuntimeError("k_residual and v_residual must hold the same number of tokens")
+        R = k_residual.shape[1]
+        keep += [k_residual, v_residual]
+        a.k_res, a.v_res = k_residual.data_ptr(), v_residual.data_ptr()
+        a.kres_stride_b, a.kres_stride_t, a.kres_stride_h = (k_residual.stride(0), k_residual.stride(1),
+                                                               k_residual.stride(2))
+        a.vres_stride_b, a.vres_stride_t, a.vres_stride_h = (v_residual.stride(0), v_residual.stride(1),
+                                                               v_residual.stride(2))
+        if isinstance(residual_len, torch.Tensor):
+            keep.append(_i32_dev(residual_len, b, device, "residual_len"))
+            a.res_lens = residual_len.data_ptr()
+            a.res_len = R
+            a.max_res_len = R if max_residual_len is None else int(max_residual_len)
+        else:
+            a.res_len = R if residual_len is None else int(residual_len)
+            a.max_res_len = a.res_len
+        if a.max_res_len > R or a.res_len > R or a.res_len < 0:
+            raise RuntimeError("residual_len exceeds the residual window")
+    elif residual_len is not None:
+        raise RuntimeError("residual_len given without k_residual / v_residual")
+
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        if out.shape != q.shape or out.dtype != q.dtype or out.device != device or out.stride(3) != 1:
+            raise RuntimeError("out must match q in shape, dtype and device")
+    keep.append(out)
+    a.out, a.out_stride_b, a.out_stride_h = out.data_ptr(), out.stride(0), out.stride(2)
+    lse = None
+    if return_lse:
+        lse = torch.empty((b, h), dtype=torch.float32, device=device)
+        keep.append(lse)
+        a.softmax_lse = lse.data_ptr()
+    a.b, a.h, a.h_k, a.d = b, h, h_k, d
+    a.bits, a.group_size, a.dtype = num_bits, group_size, dtype
+    a.softmax_scale = float(softmax_scale)
+    L = _lib.lib()
+    with torch.cuda.device(device):
+        ns = int(num_splits)
+        if ns == 0:
+            ns = L.bitdecode_num_splits(b, h_k, a.max_seqlen_k, a.max_res_len, 0)
+        a.num_splits = ns
+        nbytes = L.bitdecode_fwd_workspace_bytes(b, h, ns)
+        if nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            keep.append(ws)
+            a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
+    return DecodePlan(a, out, lse, tuple(keep), device)
+
+
+def fwd_kvcache_int(q: torch.Tensor,
+                    k_pack: torch.Tensor, k_params: torch.Tensor,
+                    v_pack: torch.Tensor, v_params: torch.Tensor,
+                    opt_block_table: Optional[torch.Tensor] = None,
+                    softmax_scale: float = 1.0,
+                    quant_mode: str = "k-channel",
+                    group_size: int = 128,
+                    num_bits: int = 4,
+                    **kwargs):
+    """Decode attention of one query token per sequence over the packed cache
+    (reference: bit_decode_interface.py:43-86; non-causal, no softcap, heuristic split count).
+
+    q [b, 1, h, 128] fp16/bf16; returns a new tensor of the same shape.  `softmax_scale`
+    defaults to 1.0 as in the reference; callers pass 1/sqrt(d).
+
+    Keyword-only extensions:
+      seqlen_k          valid packed tokens (multiple of 128); default = capacity of the cache
+      seqlens_k         int32 [b] device tensor of per-sequence packed lengths (ragged batch)
+      max_seqlen_k      host upper bound of seqlens_k (default: capacity)
+      k_residual, v_residual   fp16 window of recent tokens [b, R, h_k, 128], attended after the
+                        packed prefix; residual_len = valid tokens (int or int32 [b] tensor)
+      num_splits        0 = choose; out = preallocated output; return_lse -> (out, lse [b, h])
+    """
+    return_lse = kwargs.get("return_lse", False)
+    plan = plan_fwd_kvcache_int(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale,
+                                quant_mode, group_size, num_bits, **kwargs)
+    with torch.cuda.device(plan.device):
+        plan.run()
+    return (plan.out, plan.lse) if return_lse else plan.out

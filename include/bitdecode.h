@@ -1,0 +1,110 @@
+/* C ABI of the MI355X low-bit KV-cache decode library (libbitdecode.so).
+ *
+ * These entry points are what the reference's Python package binds for this path through
+ * its pybind module `bit_decode_cuda` (csrc/bit_decode/decode_api.cpp:605-611):
+ *   kvcache_pack_i2/_i4  ->  bitdecode_qpack
+ *   fwd_kvcache_i2/_i4   ->  bitdecode_fwd
+ * All pointers are device pointers unless stated; strides are in elements; every call is
+ * asynchronous on `stream` (a hipStream_t passed as void*), keeps no state between calls
+ * and returns 0 on success or a BITDECODE_E* code (no exceptions cross the boundary;
+ * bitdecode_last_error() gives the message for the calling thread).
+ */
+#ifndef BITDECODE_H_
+#define BITDECODE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BITDECODE_ABI_VERSION 1
+
+enum {
+    BITDECODE_OK = 0,
+    BITDECODE_EINVAL = 1,      /* bad argument (shape, divisibility, null pointer)        */
+    BITDECODE_EUNSUPPORTED = 2,/* valid request the kernels do not implement              */
+    BITDECODE_EWORKSPACE = 3,  /* workspace too small                                     */
+    BITDECODE_ELAUNCH = 4      /* HIP reported an error at launch                         */
+};
+
+enum { BITDECODE_FP16 = 0, BITDECODE_BF16 = 1 };
+
+/* Quantize-pack n_tokens new tokens of K and V into the packed cache.
+ * Replaces kvcache_qpack<num_bits> (csrc/bit_decode/decode_api.cpp:517-603) and the kernel it
+ * launches (csrc/bit_decode/src/flash_fwd_kernel.h:732-1091).  K is quantized per channel over
+ * groups of group_size consecutive tokens, V per token over groups of group_size consecutive
+ * channels; scale and zero (= group minimum) are stored in the element type. */
+typedef struct bitdecode_qpack_args {
+    const void* k;             /* [b, n_tokens, h_k, 128] fp16/bf16, last dim contiguous    */
+    const void* v;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    void* k_pack;              /* caller-allocated, reference shapes (see layout)           */
+    void* k_params;
+    void* v_pack;
+    void* v_params;
+    int32_t b, n_tokens, h_k, d;   /* d must be 128; n_tokens a multiple of 128            */
+    int32_t cache_tokens;      /* capacity S of the packed tensors, multiple of 128         */
+    int32_t dst_offset;        /* token offset of the first written chunk (multiple of 128) */
+    const int32_t* dst_offsets;/* optional device int32[b]: per-sequence dst offset         */
+    int32_t bits;              /* 2 or 4                                                    */
+    int32_t group_size;        /* 32, 64 or 128                                             */
+    int32_t dtype;             /* BITDECODE_FP16 / BITDECODE_BF16                           */
+} bitdecode_qpack_args;
+
+int bitdecode_qpack(const bitdecode_qpack_args* args, void* stream);
+
+/* Decode attention of one query token per sequence over [packed prefix || fp16 residual].
+ * Replaces mha_fwd_kvcache<num_bits> (csrc/bit_decode/decode_api.cpp:301-441), the split-KV
+ * kernel (flash_fwd_kernel.h:66-728) and the combine kernel (flash_fwd_kernel.h:1144-1327). */
+typedef struct bitdecode_fwd_args {
+    const void* q;             /* [b, 1, h, 128], last dim contiguous                       */
+    int64_t q_stride_b, q_stride_h;
+    const void* k_pack;
+    const void* k_params;
+    const void* v_pack;
+    const void* v_params;
+    int32_t cache_tokens;      /* capacity S of the packed tensors                          */
+    int32_t seqlen_k;          /* valid packed tokens (multiple of 128), all sequences      */
+    const int32_t* seqlens_k;  /* optional device int32[b] overriding seqlen_k              */
+    const void* k_res;         /* optional fp16/bf16 residual window [b, R, h_k, 128]       */
+    const void* v_res;
+    int64_t kres_stride_b, kres_stride_t, kres_stride_h;
+    int64_t vres_stride_b, vres_stride_t, vres_stride_h;
+    int32_t res_len;           /* valid residual tokens, all sequences                      */
+    const int32_t* res_lens;   /* optional device int32[b] overriding res_len               */
+    int32_t max_seqlen_k;      /* upper bound of seqlens_k (host value, sizes the grid)     */
+    int32_t max_res_len;       /* upper bound of res_lens                                   */
+    void* out;                 /* [b, 1, h, 128] element type of q                          */
+    int64_t out_stride_b, out_stride_h;
+    float* softmax_lse;        /* optional [b, h] natural-log LSE                           */
+    void* workspace;           /* >= bitdecode_fwd_workspace_bytes(...) or NULL if 1 split  */
+    size_t workspace_bytes;
+    int32_t b, h, h_k, d;      /* d must be 128, h % h_k == 0, h / h_k <= 8                 */
+    int32_t bits, group_size, dtype;
+    float softmax_scale;
+    int32_t num_splits;        /* 0 = choose (bitdecode_num_splits)                         */
+} bitdecode_fwd_args;
+
+int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
+
+/* Split count the library would choose for this problem (host function, no GPU work);
+ * replaces num_splits_heuristic (csrc/bit_decode/decode_api.cpp:234-268), retuned for 256 CUs.
+ * num_cus <= 0 queries the current device. */
+int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
+                         int32_t num_cus);
+
+/* Workspace the split path needs: fp32 partial outputs and LSEs
+ * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,
+ * csrc/bit_decode/decode_api.cpp:292-295). */
+size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits);
+
+int bitdecode_abi_version(void);
+const char* bitdecode_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITDECODE_H_ */

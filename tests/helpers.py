@@ -1,0 +1,72 @@
+"""Shared test plumbing: numpy oracle <-> torch device tensors."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from oracle import bitdecode_oracle as O
+
+
+def torch_dtype(dtype: str):
+    return torch.float16 if dtype == "fp16" else torch.bfloat16
+
+
+def to_dev(x: np.ndarray, dtype: str, device) -> torch.Tensor:
+    """fp32 numpy holding storage-representable values -> device tensor of that dtype."""
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch_dtype(dtype)).to(device)
+
+
+def bits16(x: np.ndarray, dtype: str) -> np.ndarray:
+    """fp32 values representable in dtype -> their 16-bit patterns."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if dtype == "fp16":
+        return x.astype(np.float16).view(np.uint16)
+    return (x.view(np.uint32) >> 16).astype(np.uint16)
+
+
+def alloc_cache(b, S, h_k, bits, gs, device, fill=None):
+    """Caller-side allocation with the reference's shapes (evaluation/test.py:74-83)."""
+    pn = 16 // bits
+    d = 128
+    mk = torch.zeros if fill is None else (lambda *a, **k: torch.full(*a, fill_value=fill, **k))
+    k_pack = mk((b, S // pn, h_k, d), dtype=torch.uint16, device=device)
+    k_params = torch.zeros((b, S // gs, h_k, d), dtype=torch.float32, device=device)
+    v_pack = mk((b, S, h_k, d // pn), dtype=torch.uint16, device=device)
+    v_params = torch.zeros((b, d // gs, h_k, S), dtype=torch.float32, device=device)
+    return k_pack, k_params, v_pack, v_params
+
+
+def cache_to_numpy(k_pack, k_params, v_pack, v_params):
+    return (k_pack.cpu().view(torch.int16).numpy().view(np.uint16),
+            k_params.cpu().numpy(),
+            v_pack.cpu().view(torch.int16).numpy().view(np.uint16),
+            v_params.cpu().numpy())
+
+
+def cache_from_numpy(arrs, device):
+    kp, kpar, vp, vpar = arrs
+    return (torch.from_numpy(kp.view(np.int16).copy()).view(torch.uint16).to(device),
+            torch.from_numpy(kpar.copy()).to(device),
+            torch.from_numpy(vp.view(np.int16).copy()).view(torch.uint16).to(device),
+            torch.from_numpy(vpar.copy()).to(device))
+
+
+def oracle_physical(qkv: O.QuantKV):
+    """Quantizer-oracle output laid out in the physical format (host-side packing)."""
+    from bitladder_amd import layout as L
+    dt = qkv.dtype
+    return L.pack_physical(qkv.k_codes, bits16(qkv.k_scale, dt), bits16(qkv.k_zero, dt),
+                           qkv.v_codes, bits16(qkv.v_scale, dt), bits16(qkv.v_zero, dt),
+                           qkv.bits, qkv.group_size)
+
+
+def assert_cache_equals_oracle(cache_np, qkv: O.QuantKV):
+    from bitladder_amd import layout as L
+    dt = qkv.dtype
+    kc, ks, kz, vc, vs, vz = L.unpack_physical(*cache_np, qkv.bits, qkv.group_size)
+    np.testing.assert_array_equal(kc, qkv.k_codes, err_msg="K codes")
+    np.testing.assert_array_equal(vc, qkv.v_codes, err_msg="V codes")
+    np.testing.assert_array_equal(ks, bits16(qkv.k_scale, dt), err_msg="K scale")
+    np.testing.assert_array_equal(kz, bits16(qkv.k_zero, dt), err_msg="K zero")
+    np.testing.assert_array_equal(vs, bits16(qkv.v_scale, dt), err_msg="V scale")
+    np.testing.assert_array_equal(vz, bits16(qkv.v_zero, dt), err_msg="V zero")

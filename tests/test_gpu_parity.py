@@ -1,0 +1,102 @@
+"""GPU parity tests: HIP kernels (through the C ABI) against the CPU oracle.
+
+Bars: packed codes and scale/zero bit-exact; attention output within 2e-3 max-abs of
+dequantize-then-attend computed in fp32.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import bitdecode_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-3
+SCALE = 1.0 / math.sqrt(128)
+
+
+def _pack_gpu(k, v, bits, gs, dtype, device, S):
+    from bitladder_amd import kvcache_pack_int
+    b, _, h_k, _ = k.shape
+    cache = H.alloc_cache(b, S, h_k, bits, gs, device)
+    kd, vd = H.to_dev(k[:, :S], dtype, device), H.to_dev(v[:, :S], dtype, device)
+    cu = torch.arange(0, (b + 1) * S, S, dtype=torch.int32, device=device)
+    kvcache_pack_int(kd, cache[0], cache[1], vd, cache[2], cache[3], None, cu, S, "k-channel", gs, bits)
+    return cache
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("bits", [2, 4])
+def test_qpack_bit_exact(device, bits, gs, dtype):
+    b, h_k, S = 2, 3, 384
+    q, k, v = O.make_inputs(b, h_k, h_k, S, 0, seed=bits * 100 + gs, dtype=dtype)
+    # edge groups: constant K group, constant V group, max-range values, exact .5 ties
+    k[0, :gs, 0, 5] = 1.5
+    v[0, 7, 1, :gs] = -2.25
+    k[1, gs:2 * gs, 1, 9] = np.linspace(-3, 3, gs, dtype=np.float32)
+    v[1, 3, 2, :] = 0.0
+    k[0, 0, 2, 17], k[0, 1, 2, 17] = 65504.0, -65504.0
+    k, v = O.round_to_storage(k, dtype), O.round_to_storage(v, dtype)
+    want = O.quantize_kv_ref(k, v, bits, gs, dtype)
+    cache = _pack_gpu(k, v, bits, gs, dtype, device, S)
+    torch.cuda.synchronize()
+    H.assert_cache_equals_oracle(H.cache_to_numpy(*cache), want)
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 128), (4, 32), (2, 128), (2, 64), (4, 64), (2, 32)])
+@pytest.mark.parametrize("h,h_k", [(4, 4), (8, 2), (8, 1)])
+def test_decode_from_host_packed_cache(device, bits, gs, h, h_k):
+    """Decode kernel alone: the cache is laid out on the host from the quantizer oracle."""
+    from bitladder_amd import fwd_kvcache_int
+    b, S = 2, 1024
+    q, k, v = O.make_inputs(b, h, h_k, S, 0, seed=7)
+    qkv = O.quantize_kv_ref(k, v, bits, gs)
+    cache = H.cache_from_numpy(H.oracle_physical(qkv), device)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, want_lse = O.attend_ref(q, k_hat, v_hat, SCALE)
+    for ns in (0, 1, 3):
+        out, lse = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits,
+                                   num_splits=ns, return_lse=True)
+        err = np.abs(out.float().cpu().numpy() - want).max()
+        assert err < ATOL, (ns, err)
+        np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("res_len", [0, 1, 31, 32, 33, 100, 128])
+@pytest.mark.parametrize("bits,gs", [(4, 128), (2, 64)])
+def test_decode_with_residual_window(device, bits, gs, res_len):
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, S, R = 2, 8, 2, 512, 128
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=11)
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    rl = np.full(b, res_len, np.int32)
+    want, _ = O.attend_ref(q, k_hat, v_hat, SCALE, k[:, S:], v[:, S:], res_lens=rl)
+    kres, vres = H.to_dev(k[:, S:], "fp16", device), H.to_dev(v[:, S:], "fp16", device)
+    # poison the invalid tail: it must not be read into the result
+    kres[:, res_len:] = float("nan")
+    vres[:, res_len:] = float("nan")
+    out = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits,
+                          k_residual=kres, v_residual=vres, residual_len=res_len)
+    err = np.abs(out.float().cpu().numpy() - want).max()
+    assert err < ATOL, err
+
+
+def test_decode_residual_only(device):
+    """No packed prefix at all: the fp16 path alone (also the fp16-KV baseline kernel)."""
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, R = 2, 8, 2, 1000
+    q, k, v = O.make_inputs(b, h, h_k, 0, R, seed=5)
+    want, _ = O.attend_ref(q, None, None, SCALE, k, v)
+    cache = H.alloc_cache(b, 128, h_k, 4, 128, device)
+    for ns in (0, 1, 5):
+        out = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", 128, 4,
+                              seqlen_k=0, k_residual=H.to_dev(k, "fp16", device),
+                              v_residual=H.to_dev(v, "fp16", device), num_splits=ns)
+        err = np.abs(out.float().cpu().numpy() - want).max()
+        assert err < ATOL, (ns, err)
