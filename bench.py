@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the low-bit KV-cache decode step on one MI355X.
+
+A step is one decode-attention call (split-KV kernel + combine) over one batch of synthetic
+input.  Workload = Llama-3-8B-shape GQA decode: batch 1, 32 q heads / 8 kv heads, head_dim 128,
+32768 packed tokens at 4 bits (group 128) plus a 128-token fp16 residual window.
+Prints ONE JSON line; see --help for the side measurements it carries.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (b, h, h_k, S, R, bits, gs, dtype)
+    "llama3-8b-gqa-32k-4bit-g128": (1, 32, 8, 32768, 128, 4, 128, torch.float16),
+    "llama2-7b-mha-4k-4bit-g128": (1, 32, 32, 4096, 128, 4, 128, torch.float16),
+    "llama3-8b-gqa-128k-2bit-g64": (1, 32, 8, 131072, 128, 2, 64, torch.float16),
+    "llama3-70b-gqa-64k-2bit-g128-b8": (8, 64, 8, 65536, 128, 2, 128, torch.bfloat16),
+}
+
+
+def make_inputs(b, h, h_k, n_tokens, seed, dtype):
+    """Seeded N(0,1) on the CPU (so a CPU checker sees the same bits); 3 of 128 K channels per
+    kv-head are multiplied by 10 (2 % outlier channels)."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((b, 1, h, 128), generator=g)
+    k = torch.randn((b, n_tokens, h_k, 128), generator=g)
+    v = torch.randn((b, n_tokens, h_k, 128), generator=g)
+    for hk in range(h_k):
+        ch = torch.randperm(128, generator=g)[:3]
+        k[:, :, hk, ch] *= 10.0
+    return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+def algorithmic_bytes(b, h, h_k, S, R, bits, gs):
+    packed = b * h_k * S * 128 * 2 * (bits / 8 + 4 / gs)
+    resid = b * h_k * R * 128 * 2 * 2
+    qo = 2 * b * h * 128 * 2
+    return int(packed + resid + qo), int(packed)
+
+
+def alloc_cache(b, S, h_k, bits, gs, dev):
+    pn = 16 // bits
+    return (torch.zeros((b, S // pn, h_k, 128), dtype=torch.uint16, device=dev),
+            torch.zeros((b, S // gs, h_k, 128), dtype=torch.float32, device=dev),
+            torch.zeros((b, S, h_k, 128 // pn), dtype=torch.uint16, device=dev),
+            torch.zeros((b, 128 // gs, h_k, S), dtype=torch.float32, device=dev))
+
+
+def time_steps(run_step, steps, warmup, use_graph):
+    """Returns (wall seconds, event seconds) for exactly `steps` steps."""
+    dev = torch.device("cuda:0")
+    for i in range(warmup):
+        run_step(i)
+    torch.cuda.synchronize(dev)
+    graph = None
+    if use_graph:
+        try:
+            side = torch.cuda.Stream(dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):
+                run_step(0)
+            torch.cuda.current_stream(dev).wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(steps):
+                    run_step(i)
+            graph.replay()          # untimed: first replay uploads the graph
+            torch.cuda.synchronize(dev)
+        except Exception as e:      # noqa: BLE001
+            print(f"[bench] graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
+            graph = None
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    e0.record()
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(steps):
+            run_step(i)
+    e1.record()
+    torch.cuda.synchronize(dev)
+    t1 = time.perf_counter()
+    return t1 - t0, e0.elapsed_time(e1) * 1e-3, graph is not None
+
+
+def cpu_baseline(q, k, v, S, R, bits, gs, scale, budget_s=20.0):
+    """Reference semantics on the host cores: the torch oracle (dequantize the packed cache to
+    fp32, fp32 softmax attention over [packed || residual]) timed on the same inputs."""
+    from oracle import torch_oracle as TO
+    torch.set_num_threads(os.cpu_count() or 1)
+    qkv = TO.quantize_kv(k[:, :S].float(), v[:, :S].float(), bits, gs, k.dtype)
+    fn = lambda: TO.dequant_attend(q.float(), qkv, scale, k[:, S:].float(), v[:, S:].float())
+    fn()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 50):
+        t0 = time.perf_counter()
+        out = fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return out, times[len(times) // 2], len(times)
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="llama3-8b-gqa-32k-4bit-g128", choices=sorted(WORKLOADS))
+    ap.add_argument("--num-splits", type=int, default=0)
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of one HIP graph")
+    ap.add_argument("--no-rotate", action="store_true", help="reuse one KV cache (stays in the 256 MB Infinity Cache)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-fp16", action="store_true", help="skip the fp16-KV baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this decode path has no cross-GPU step (it shards by kv-head / batch "
+              "with no exchange); run with --gpus 1", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+
+    from bitladder_amd import kvcache_pack_int, plan_fwd_kvcache_int
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    b, h, h_k, S, R, bits, gs, dtype = WORKLOADS[args.workload]
+    scale = 1.0 / math.sqrt(128)
+    total_bytes, packed_bytes = algorithmic_bytes(b, h, h_k, S, R, bits, gs)
+
+    # enough distinct caches that consecutive steps cannot be served from the Infinity Cache
+    nbuf = 1 if args.no_rotate else max(2, math.ceil(320e6 / total_bytes))
+    nbuf = min(nbuf, 16)
+    plans, keep = [], []
+    q0 = k0 = v0 = None
+    for i in range(nbuf):
+        q, k, v = make_inputs(b, h, h_k, S + R, seed=i, dtype=dtype)
+        if i == 0:
+            q0, k0, v0 = q, k, v
+        kd, vd = k.to(dev), v.to(dev)
+        cache = alloc_cache(b, S, h_k, bits, gs, dev)
+        kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S,
+                         "k-channel", gs, bits)
+        kres, vres = kd[:, S:].contiguous(), vd[:, S:].contiguous()
+        plan = plan_fwd_kvcache_int(q.to(dev), *cache, None, scale, "k-channel", gs, bits,
+                                    k_residual=kres, v_residual=vres, num_splits=args.num_splits)
+        plans.append(plan)
+        keep.append((cache, kres, vres))
+        del kd, vd
+    torch.cuda.synchronize(dev)
+
+    def step(i):
+        plans[i % nbuf].run()
+
+    wall, evs, graphed = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    us_step = wall / args.steps * 1e6
+    us_step_ev = evs / args.steps * 1e6
+    achieved = total_bytes / (us_step_ev * 1e-6) / 1e9
+
+    result = {
+        "metric": "us/decode step (+ HBM GB/s, % of peak), Llama-3-8B GQA, 4-bit KV @32K ctx"
+                  if args.workload.startswith("llama3-8b-gqa-32k") else f"us/decode step, {args.workload}",
+        "value": round(us_step, 3),
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_step * 1e-3, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16" if dtype == torch.float16 else "bf16",
+        "data": "synthetic: seeded N(0,1) q/k/v, 3 of 128 K channels per kv-head x10, packed by the library's own "
+                "quantize-pack kernel",
+        "config": {"workload": args.workload, "batch": b, "q_heads": h, "kv_heads": h_k, "head_dim": 128,
+                   "packed_tokens": S, "residual_tokens": R, "bits": bits, "group_size": gs,
+                   "num_splits": plans[0].num_splits, "kv_buffers_rotated": nbuf,
+                   "launch": "hip-graph" if graphed else "eager"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "fwd_splitkv_kernel", "algorithmic_bytes": total_bytes,
+                     "packed_stream_bytes": packed_bytes, "us_per_step_events": round(us_step_ev, 3)},
+    }
+
+    if not args.no_fp16:
+        # fp16-KV decode on the same GPU: the library's own fp16 split-KV path over all S+R tokens,
+        # and torch SDPA for comparison
+        fplans = []
+        nb16 = 1 if args.no_rotate else max(2, min(8, math.ceil(320e6 / (b * h_k * (S + R) * 512))))
+        dummy = alloc_cache(b, 128, h_k, bits, gs, dev)
+        for i in range(nb16):
+            q, k, v = make_inputs(b, h, h_k, S + R, seed=100 + i, dtype=dtype)
+            kd, vd = k.to(dev), v.to(dev)
+            fplans.append((plan_fwd_kvcache_int(q.to(dev), *dummy, None, scale, "k-channel", gs, bits, seqlen_k=0,
+                                                k_residual=kd, v_residual=vd), q.to(dev), kd, vd))
+        torch.cuda.synchronize(dev)
+        w16, e16, _ = time_steps(lambda i: fplans[i % nb16][0].run(), args.steps, args.warmup, not args.no_graph)
+        us16 = e16 / args.steps * 1e6
+        fp16_bytes = b * h_k * (S + R) * 128 * 2 * 2 + 2 * b * h * 128 * 2
+
+        def sdpa(i):
+            _, qd, kd, vd = fplans[i % nb16]
+            torch.nn.functional.scaled_dot_product_attention(
+                qd.transpose(1, 2), kd.transpose(1, 2), vd.transpose(1, 2), scale=scale, enable_gqa=True)
+        try:
+            _, es, _ = time_steps(sdpa, max(10, args.steps // 4), 3, False)
+            us_sdpa = es / max(10, args.steps // 4) * 1e6
+        except Exception as e:  # noqa: BLE001
+            print(f"[bench] torch SDPA baseline failed: {e}", file=sys.stderr)
+            us_sdpa = None
+        result["fp16_kv_baseline"] = {
+            "us_per_step": round(us16, 3), "GB/s": round(fp16_bytes / (us16 * 1e-6) / 1e9, 1),
+            "kernel": "same library, fp16 split-KV path", "speedup_of_low_bit": round(us16 / us_step_ev, 3),
+            "torch_sdpa_us_per_step": None if us_sdpa is None else round(us_sdpa, 3)}
+        del fplans
+
+    if not args.no_cpu:
+        out_cpu, t_cpu, reps = cpu_baseline(q0, k0, v0, S, R, bits, gs, scale)
+        out_gpu = plans[0].run().float().cpu()
+        torch.cuda.synchronize(dev)
+        result["cpu_baseline"] = {
+            "value": round(t_cpu * 1e6, 1), "unit": "us/step", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"full {args.workload} decode step (dequantize to fp32 + fp32 attention incl. residual), "
+                      f"median of {reps} runs, torch CPU ops on {torch.get_num_threads()} threads "
+                      f"(os.cpu_count()={os.cpu_count()})",
+            "max_abs_err_gpu_vs_cpu": float((out_gpu - out_cpu).abs().max())}
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

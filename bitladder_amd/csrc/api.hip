@@ -43,23 +43,23 @@ int query_cus() {
     return n;
 }
 
-// One wave handles one work unit (a 128-token packed chunk or a 32-token fp16 block) at a time and
-// a workgroup has 8 waves.  Pick the number of splits so that the whole grid is about one
-// workgroup per CU while every wave still gets at least one unit.
-int choose_splits(int b, int hk, int max_units, int num_cus) {
-    if (max_units <= 0) return 1;
+// A wave streams whole 128-token packed chunks (plus a share of the 16-token fp16 tiles) and a
+// workgroup has 8 waves.  Pick the number of splits so that the grid is about one workgroup per CU
+// while every wave still gets at least one chunk (or four fp16 tiles when nothing is packed).
+int choose_splits(int b, int hk, int max_seqlen_k, int max_res_len, int num_cus) {
+    const int chunks = max_seqlen_k / bitdecode::kChunk;
+    const int tiles = (max_res_len + 15) / 16;
+    const int units = chunks > 0 ? chunks : (tiles + 3) / 4;
+    if (units <= 0) return 1;
     const int heads = std::max(1, b * hk);
     const int by_occupancy = std::max(1, (num_cus + heads - 1) / heads);
-    const int by_work = std::max(1, (max_units + 7) / 8);
-    int n = std::min(by_occupancy, by_work);
-    n = std::min(n, 256);
+    const int by_work = std::max(1, (units + 7) / 8);
+    int n = std::min(std::min(by_occupancy, by_work), 256);
     // drop splits that would be empty: ceil(units / n) units per split
-    const int ups = (max_units + n - 1) / n;
-    n = (max_units + ups - 1) / ups;
+    const int ups = (units + n - 1) / n;
+    n = (units + ups - 1) / ups;
     return std::max(1, n);
 }
-
-int units_of(int seqlen_k, int res_len) { return seqlen_k / bitdecode::kChunk + (res_len + 31) / 32; }
 
 }  // namespace
 
@@ -71,12 +71,15 @@ const char* bitdecode_last_error(void) { return g_err; }
 
 int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len, int32_t num_cus) {
     if (num_cus <= 0) num_cus = query_cus();
-    return choose_splits(b, h_k, units_of(max_seqlen_k, max_res_len), num_cus);
+    return choose_splits(b, h_k, max_seqlen_k, max_res_len, num_cus);
 }
+
+// [tickets: b*h ints rounded up to 256 B][o_part][lse_part]
+static size_t ticket_bytes(int32_t b, int32_t h) { return (static_cast<size_t>(b) * h * sizeof(int) + 255) / 256 * 256; }
 
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     if (num_splits <= 1) return 0;
-    return static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 1) * sizeof(float);
+    return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 1) * sizeof(float);
 }
 
 int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
@@ -157,7 +160,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
 
     int nsplit = a->num_splits;
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
-    if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, units_of(max_s, max_r), query_cus());
+    if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus());
     if (nsplit > 1) {
         const size_t need = bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
         if (!a->workspace || a->workspace_bytes < need)
@@ -191,7 +194,8 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     P.scale_log2 = a->softmax_scale * 1.4426950408889634f;   // decode_api.cpp:128-142
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
     if (nsplit > 1) {
-        P.o_part = static_cast<float*>(a->workspace);
+        P.tickets = static_cast<int*>(a->workspace);
+        P.o_part = reinterpret_cast<float*>(static_cast<uint8_t*>(a->workspace) + ticket_bytes(a->b, a->h));
         P.lse_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
     }
     hipError_t e = launch_fwd(P, static_cast<hipStream_t>(stream));

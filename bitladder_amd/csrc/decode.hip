@@ -24,7 +24,8 @@
 //    the same MFMA and are added afterwards with one row-rotate (lane ^ 8) per accumulator.
 //  * Online softmax in base 2 per head (softmax.h:250-310), running max shared by the four
 //    lanes of a head through two cross-lane exchanges, row sums kept per lane until the end.
-//  * The waves of a workgroup merge through LDS, splits merge in the combine kernel.
+//  * The waves of a workgroup merge through LDS; splits merge in the same launch: the workgroup
+//    that draws the last ticket of a (batch, kv-head) combines all partials.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -177,35 +178,89 @@ __device__ __forceinline__ void softmax_step(float (&s)[N], WaveState<NCG>& st) 
 }
 
 // ---------------------------------------------------------------------------------------------
-// one packed 128-token chunk
+// packed 128-token chunks
 // ---------------------------------------------------------------------------------------------
+// Registers holding one chunk's global loads.  K side and V side are separate so that the next
+// chunk's K loads can be issued as soon as this chunk's K registers are consumed (and likewise
+// for V): with one chunk per wave every load of the kernel is in flight from the first cycle.
+template <int BITS, int GS>
+struct KSide {
+    static constexpr int NG = kChunk / GS;
+    static constexpr int NW4 = BITS == 4 ? 8 : 4;     // 16-byte lane loads of codes per chunk
+    static constexpr int PF = NG <= 2 ? NG : 1;       // parameter groups fetched with the chunk
+    u4 code[NW4];
+    u4 ps[PF][4], pz[PF][4];
+};
+template <int BITS, int GS>
+struct VSide {
+    static constexpr int NCG = kHeadDim / GS;
+    static constexpr int NW4 = BITS == 4 ? 8 : 4;
+    static constexpr int PF = NCG == 1 ? 4 : 0;       // sub-blocks whose params are fetched with the chunk
+    u4 code[NW4];
+    u4 ps[PF ? PF : 1], pz[PF ? PF : 1];
+};
+
+template <int BITS, int GS>
+__device__ __forceinline__ void load_kside(KSide<BITS, GS>& K, const FwdParams& P, int64_t bh, int ci, int lane) {
+    constexpr int NG = kChunk / GS;
+    const int kg = lane >> 4;
+    const uint8_t* kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
+    const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
+#pragma unroll
+    for (int g = 0; g < KSide<BITS, GS>::PF; ++g) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            K.ps[g][j] = ld_u4(kp + g * kKParamGroupBytes + (32 * j + 8 * kg) * 2);
+            K.pz[g][j] = ld_u4(kp + g * kKParamGroupBytes + 256 + (32 * j + 8 * kg) * 2);
+        }
+    }
+#pragma unroll
+    for (int x = 0; x < KSide<BITS, GS>::NW4; ++x) K.code[x] = ld_u4(kc + x * 1024 + lane * 16);
+}
+
+template <int BITS, int GS>
+__device__ __forceinline__ void load_vside(VSide<BITS, GS>& V, const FwdParams& P, int64_t bh, int ci, int lane) {
+    const int kg = lane >> 4;
+    const uint8_t* vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
+    const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
+#pragma unroll
+    for (int sb = 0; sb < VSide<BITS, GS>::PF; ++sb) {
+        V.ps[sb] = ld_u4(vp + sb * 128 + kg * 16);
+        V.pz[sb] = ld_u4(vp + sb * 128 + 64 + kg * 16);
+    }
+#pragma unroll
+    for (int x = 0; x < VSide<BITS, GS>::NW4; ++x) V.code[x] = ld_u4(vc + x * 1024 + lane * 16);
+}
+
+// S^T = K Q^T for the 8 tiles of a chunk, then the online-softmax step.  On return s[] holds
+// the probabilities 2^kPShift * exp2(score - running max) of this lane's 32 tokens.
 template <int BITS, int GS, bool BF16>
-__device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int ci, int lane,
-                                             const h8 (&qB)[4], bool lo_part,
+__device__ __forceinline__ void chunk_scores(const KSide<BITS, GS>& K, const FwdParams& P, int64_t bh, int ci,
+                                             int lane, const h8 (&qB)[4], bool lo_part, float (&s)[32],
                                              WaveState<kHeadDim / GS>& st) {
     constexpr int NG = kChunk / GS;
     constexpr int NCG = kHeadDim / GS;
     constexpr int TPG = GS / 16;      // 16-token tiles per K group
-    constexpr int CTPG = GS / 16;     // 16-channel tiles per V channel group
+    constexpr int PF = KSide<BITS, GS>::PF;
     const int kg = lane >> 4;
     const h8 off = code_offsets<BITS>();
-    const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
-
-    const uint8_t* kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
     const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
-    const uint8_t* vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
-    const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
 
-    // ---- S^T = K Q^T for the 8 tiles of the chunk
-    float s[32];
 #pragma unroll
     for (int grp = 0; grp < NG; ++grp) {
         h8 qp[4];
         float kap = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const h8 sc = ld_h8<BF16>(kp + grp * kKParamGroupBytes + (32 * j + 8 * kg) * 2);
-            const h8 zr = ld_h8<BF16>(kp + grp * kKParamGroupBytes + 256 + (32 * j + 8 * kg) * 2);
+            u4 rs, rz;
+            if (grp < PF) {
+                rs = K.ps[grp < PF ? grp : 0][j];
+                rz = K.pz[grp < PF ? grp : 0][j];
+            } else {
+                rs = ld_u4(kp + grp * kKParamGroupBytes + (32 * j + 8 * kg) * 2);
+                rz = ld_u4(kp + grp * kKParamGroupBytes + 256 + (32 * j + 8 * kg) * 2);
+            }
+            const h8 sc = cvt_h8<BF16>(rs), zr = cvt_h8<BF16>(rz);
             qp[j] = split_mul(qB[j], sc, lo_part);
             if (!lo_part) kap = dot8(qB[j], zr, kap);
             kap = -dot8(qp[j], off, -kap);
@@ -215,7 +270,7 @@ __device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int
 #pragma unroll
             for (int tt = 0; tt < TPG; ++tt) {
                 const int t = grp * TPG + tt;
-                const u4 w = ld_u4(kc + t * 1024 + lane * 16);
+                const u4 w = K.code[t];
                 f4 acc = {0, 0, 0, 0};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc = mfma32(dq4(w[j]), qp[j], acc);
@@ -229,7 +284,7 @@ __device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int
 #pragma unroll
             for (int pp = 0; pp < TPG / 2; ++pp) {
                 const int tp = grp * (TPG / 2) + pp;
-                const u4 w = ld_u4(kc + tp * 1024 + lane * 16);
+                const u4 w = K.code[tp];
 #pragma unroll
                 for (int tin = 0; tin < 2; ++tin) {
                     f4 acc = {0, 0, 0, 0};
@@ -250,10 +305,21 @@ __device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int
             }
         }
     }
-
     softmax_step<32, NCG>(s, st);
+}
 
-    // ---- O^T += V^T P^T, 32 tokens (one k-step) at a time
+// O^T += V^T P^T for one chunk, 32 tokens (one k-step) at a time
+template <int BITS, int GS, bool BF16>
+__device__ __forceinline__ void chunk_pv(const VSide<BITS, GS>& V, const FwdParams& P, int64_t bh, int ci, int lane,
+                                         bool lo_part, const float (&s)[32], WaveState<kHeadDim / GS>& st) {
+    constexpr int NCG = kHeadDim / GS;
+    constexpr int CTPG = GS / 16;     // 16-channel tiles per V channel group
+    constexpr int PF = VSide<BITS, GS>::PF;
+    const int kg = lane >> 4;
+    const h8 off = code_offsets<BITS>();
+    const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
+    const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
+
     h8 p16[4];
 #pragma unroll
     for (int sb = 0; sb < 4; ++sb) {
@@ -269,15 +335,24 @@ __device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int
         st.l = dot8(p16[sb], ones, st.l);
     }
 
+    auto params = [&](int sb, int cg, h8& vs, h8& vz) {
+        if (PF) {
+            vs = cvt_h8<BF16>(V.ps[PF ? sb : 0]);
+            vz = cvt_h8<BF16>(V.pz[PF ? sb : 0]);
+        } else {
+            vs = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + kg * 16);
+            vz = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + 64 + kg * 16);
+        }
+    };
+
     if constexpr (BITS == 4) {
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
-            const u4 w0 = ld_u4(vc + sb * 2048 + lane * 16);
-            const u4 w1 = ld_u4(vc + sb * 2048 + 1024 + lane * 16);
+            const u4 w0 = V.code[2 * sb], w1 = V.code[2 * sb + 1];
 #pragma unroll
             for (int cg = 0; cg < NCG; ++cg) {
-                const h8 vs = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + kg * 16);
-                const h8 vz = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + 64 + kg * 16);
+                h8 vs, vz;
+                params(sb, cg, vs, vz);
                 const h8 pp = split_mul(p16[sb], vs, lo_part);
                 if (!lo_part) st.bv[cg] = dot8(p16[sb], vz, st.bv[cg]);
                 st.bv[cg] = -dot8(pp, off, -st.bv[cg]);
@@ -292,16 +367,15 @@ __device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int
     } else {
 #pragma unroll
         for (int sb2 = 0; sb2 < 2; ++sb2) {
-            const u4 w0 = ld_u4(vc + sb2 * 2048 + lane * 16);
-            const u4 w1 = ld_u4(vc + sb2 * 2048 + 1024 + lane * 16);
+            const u4 w0 = V.code[2 * sb2], w1 = V.code[2 * sb2 + 1];
 #pragma unroll
             for (int cg = 0; cg < NCG; ++cg) {
                 h8 pp[2];
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
                     const int sb = 2 * sb2 + ks;
-                    const h8 vs = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + kg * 16);
-                    const h8 vz = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + 64 + kg * 16);
+                    h8 vs, vz;
+                    params(sb, cg, vs, vz);
                     pp[ks] = split_mul(p16[sb], vs, lo_part);
                     if (!lo_part) st.bv[cg] = dot8(p16[sb], vz, st.bv[cg]);
                     st.bv[cg] = -dot8(pp[ks], off, -st.bv[cg]);
@@ -321,81 +395,86 @@ __device__ __forceinline__ void packed_chunk(const FwdParams& P, int64_t bh, int
 }
 
 // ---------------------------------------------------------------------------------------------
-// one 32-token block of the fp16 residual window (tokens n0 .. n0+31, valid below R)
+// 16-token tiles of the fp16 residual window (tokens n0 .. n0+15, valid below R)
 // ---------------------------------------------------------------------------------------------
-template <bool BF16, int NCG>
-__device__ __forceinline__ void fp16_block(const FwdParams& P, int bi, int hk, int n0, int R, int lane,
-                                           const h8 (&qB)[4], bool lo_part, WaveState<NCG>& st,
-                                           uint16_t* lds) {
+struct Fp16Tile {
+    u4 k[4];   // lane (token col, kg): channels 32*j + 8*kg .. +7
+    u4 v[4];   // lane (kg, col): token 4*x + kg, channels 8*col .. +7
+};
+
+__device__ __forceinline__ void load_fp16_tile(Fp16Tile& T, const FwdParams& P, int bi, int hk, int n0, int R,
+                                               int lane) {
     const int col = lane & 15, kg = lane >> 4;
-    const h8 zero8 = h8{0, 0, 0, 0, 0, 0, 0, 0};
     const uint16_t* kr = P.k_res + bi * P.kres_sb + hk * P.kres_sh;
     const uint16_t* vr = P.v_res + bi * P.vres_sb + hk * P.vres_sh;
-    const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
-
-    float s[8];
+    const int tok = n0 + col;
 #pragma unroll
-    for (int T = 0; T < 2; ++T) {
-        const int tok = n0 + 16 * T + col;
-        f4 acc = {0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            h8 a = h8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (tok < R) a = ld_h8<BF16>(kr + static_cast<int64_t>(tok) * P.kres_st + 32 * j + 8 * kg);
-            acc = mfma32(a, lo_part ? zero8 : qB[j], acc);   // fp16 operands are exact: no lo part
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int tk = n0 + 16 * T + 4 * kg + r;
-            const float sp = acc[r] * P.scale_log2;
-            const float tot = sp + partner(sp);     // outside the select: every lane must execute the DPP
-            s[4 * T + r] = tk < R ? tot : -INFINITY;
-        }
+    for (int j = 0; j < 4; ++j) {
+        T.k[j] = u4{0, 0, 0, 0};
+        if (tok < R) T.k[j] = ld_u4(kr + static_cast<int64_t>(tok) * P.kres_st + 32 * j + 8 * kg);
     }
-    softmax_step<8, NCG>(s, st);
-    h8 p16;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-        h2 t = pk_rtz(s[2 * x], s[2 * x + 1]);
-        p16[2 * x] = t[0];
-        p16[2 * x + 1] = t[1];
+        const int tv = n0 + 4 * x + kg;
+        T.v[x] = u4{0, 0, 0, 0};
+        if (tv < R) T.v[x] = ld_u4(vr + static_cast<int64_t>(tv) * P.vres_st + col * 8);
     }
-    st.l = dot8(p16, ones, st.l);
+}
+
+template <bool BF16, int NCG>
+__device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P, int n0, int R, int lane,
+                                          const h8 (&qB)[4], bool lo_part, WaveState<NCG>& st, uint16_t* lds) {
+    const int col = lane & 15, kg = lane >> 4;
+    const h8 zero8 = h8{0, 0, 0, 0, 0, 0, 0, 0};
 
     // V tile (16 tokens x 128 channels) goes through this wave's LDS slab to be read back
     // token-contiguous per channel (the MFMA A operand wants 4 tokens of one channel per lane).
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int T = 0; T < 2; ++T) {
-        __builtin_amdgcn_wave_barrier();
+    for (int x = 0; x < 4; ++x) {
+        *reinterpret_cast<u4*>(&lds[(4 * x + kg) * kLdsRowHalves + col * 8]) = T.v[x];
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    float s[4];
+    {
+        f4 acc = {0, 0, 0, 0};
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            const int tl = 4 * x + kg;
-            const int tok = n0 + 16 * T + tl;
-            u4 d = {0, 0, 0, 0};
-            if (tok < R) d = ld_u4(vr + static_cast<int64_t>(tok) * P.vres_st + col * 8);
-            *reinterpret_cast<u4*>(&lds[tl * kLdsRowHalves + col * 8]) = d;
+        for (int j = 0; j < 4; ++j) {
+            // fp16 operands are exact: only the hi columns carry q
+            acc = mfma32(cvt_h8<BF16>(T.k[j]), lo_part ? zero8 : qB[j], acc);
         }
-        __builtin_amdgcn_wave_barrier();
-        h4 pb = {p16[4 * T], p16[4 * T + 1], p16[4 * T + 2], p16[4 * T + 3]};
-        if (lo_part) pb = h4{0, 0, 0, 0};
 #pragma unroll
-        for (int ct = 0; ct < 8; ++ct) {
-            uint16_t e[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) e[i] = lds[(4 * kg + i) * kLdsRowHalves + 16 * ct + col];
-            h4 a;
-            if constexpr (BF16) {
-                h2 t0 = pk_rtz(__uint_as_float(static_cast<uint32_t>(e[0]) << 16),
-                               __uint_as_float(static_cast<uint32_t>(e[1]) << 16));
-                h2 t1 = pk_rtz(__uint_as_float(static_cast<uint32_t>(e[2]) << 16),
-                               __uint_as_float(static_cast<uint32_t>(e[3]) << 16));
-                a = h4{t0[0], t0[1], t1[0], t1[1]};
-            } else {
-                a = h4{__builtin_bit_cast(_Float16, e[0]), __builtin_bit_cast(_Float16, e[1]),
-                       __builtin_bit_cast(_Float16, e[2]), __builtin_bit_cast(_Float16, e[3])};
-            }
-            st.o[ct] = mfma16(a, pb, st.o[ct]);
+        for (int r = 0; r < 4; ++r) {
+            const int tk = n0 + 4 * kg + r;
+            const float sp = acc[r] * P.scale_log2;
+            const float tot = sp + partner(sp);     // outside the select: every lane must execute the DPP
+            s[r] = tk < R ? tot : -INFINITY;
         }
+    }
+    softmax_step<4, NCG>(s, st);
+    const h2 p01 = pk_rtz(s[0], s[1]), p23 = pk_rtz(s[2], s[3]);
+    st.l = __builtin_amdgcn_fdot2(p01, h2{1, 1}, st.l, false);
+    st.l = __builtin_amdgcn_fdot2(p23, h2{1, 1}, st.l, false);
+    h4 pb = {p01[0], p01[1], p23[0], p23[1]};
+    if (lo_part) pb = h4{0, 0, 0, 0};
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) {
+        uint16_t e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = lds[(4 * kg + i) * kLdsRowHalves + 16 * ct + col];
+        h4 a;
+        if constexpr (BF16) {
+            h2 t0 = pk_rtz(__uint_as_float(static_cast<uint32_t>(e[0]) << 16),
+                           __uint_as_float(static_cast<uint32_t>(e[1]) << 16));
+            h2 t1 = pk_rtz(__uint_as_float(static_cast<uint32_t>(e[2]) << 16),
+                           __uint_as_float(static_cast<uint32_t>(e[3]) << 16));
+            a = h4{t0[0], t0[1], t1[0], t1[1]};
+        } else {
+            a = h4{__builtin_bit_cast(_Float16, e[0]), __builtin_bit_cast(_Float16, e[1]),
+                   __builtin_bit_cast(_Float16, e[2]), __builtin_bit_cast(_Float16, e[3])};
+        }
+        st.o[ct] = mfma16(a, pb, st.o[ct]);
     }
 }
 
@@ -412,7 +491,12 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// split-KV kernel: grid (num_splits, h_k, b), kNW waves
+// split-KV kernel: grid (num_splits, h_k, b), kNW waves.
+// Split s of a (batch, kv-head) owns packed chunks [s*cps, (s+1)*cps) dealt round-robin to its
+// waves; the 16-token tiles of the fp16 window are dealt round-robin over ALL waves of the head.
+// With more than one split each workgroup writes a normalised partial and takes a ticket; the
+// workgroup that draws the last ticket of its (batch, kv-head) merges all partials
+// (flash_fwd_kernel.h:1217-1298 formula) and resets the ticket.
 // ---------------------------------------------------------------------------------------------
 template <int BITS, int GS, bool BF16>
 __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
@@ -422,6 +506,7 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
     constexpr int kLdsBytes = (kMergeFloats * 4 > kNW * kSlabHalves * 2) ? kMergeFloats * 4 : kNW * kSlabHalves * 2;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kLdsBytes];
     __shared__ float sM[kNW][kMaxGroupHeads], sL[kNW][kMaxGroupHeads];
+    __shared__ int s_last;
 
     const int split = blockIdx.x, hk = blockIdx.y, bi = blockIdx.z;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -433,10 +518,11 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
 
     const int S = P.seqlens ? P.seqlens[bi] : P.seqlen;
     const int R = P.reslens ? P.reslens[bi] : P.reslen;
-    const int nP = S / kChunk, nR = (R + 31) / 32, U = nP + nR;
-    const int ups = (U + P.nsplit - 1) / P.nsplit;
-    const int u0 = split * ups;
-    const int u1 = min(U, u0 + ups);
+    const int nP = S / kChunk;
+    const int cps = (nP + P.nsplit - 1) / P.nsplit;
+    const int c0 = min(nP, split * cps);
+    const int c1 = min(nP, c0 + cps);
+    const int nT = (R + 15) / 16;
 
     h8 qB[4];
 #pragma unroll
@@ -453,12 +539,45 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) st.o[ct] = f4{0, 0, 0, 0};
 
-    uint16_t* slab = reinterpret_cast<uint16_t*>(lds_raw) + wave * kSlabHalves;
-    for (int u = u0 + wave; u < u1; u += kNW) {
-        if (u < nP) {
-            packed_chunk<BITS, GS, BF16>(P, bh, u, lane, qB, lo_part, st);
-        } else {
-            fp16_block<BF16, NCG>(P, bi, hk, (u - nP) * 32, R, lane, qB, lo_part, st, slab);
+    // ---- packed chunks of this wave, software-pipelined one side ahead
+    {
+        int ci = c0 + wave;
+        if (ci < c1) {
+            KSide<BITS, GS> K;
+            VSide<BITS, GS> V;
+            load_kside<BITS, GS>(K, P, bh, ci, lane);
+            load_vside<BITS, GS>(V, P, bh, ci, lane);
+            while (true) {
+                float s[32];
+                chunk_scores<BITS, GS, BF16>(K, P, bh, ci, lane, qB, lo_part, s, st);
+                const int cn = ci + kNW;
+                const bool more = cn < c1;
+                if (more) load_kside<BITS, GS>(K, P, bh, cn, lane);
+                chunk_pv<BITS, GS, BF16>(V, P, bh, ci, lane, lo_part, s, st);
+                if (!more) break;
+                load_vside<BITS, GS>(V, P, bh, cn, lane);
+                ci = cn;
+            }
+        }
+    }
+    // ---- fp16 window tiles of this wave
+    {
+        uint16_t* slab = reinterpret_cast<uint16_t*>(lds_raw) + wave * kSlabHalves;
+        const int stride = kNW * P.nsplit;
+        int t = wave * P.nsplit + split;   // consecutive tiles go to different workgroups
+        if (t < nT) {
+            Fp16Tile T;
+            load_fp16_tile(T, P, bi, hk, t * 16, R, lane);
+            while (true) {
+                const int tn = t + stride;
+                Fp16Tile N;
+                const bool more = tn < nT;
+                if (more) load_fp16_tile(N, P, bi, hk, tn * 16, R, lane);
+                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, qB, lo_part, st, slab);
+                if (!more) break;
+                T = N;
+                t = tn;
+            }
         }
     }
 
@@ -466,8 +585,6 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
     st.l = colsum(st.l);
 #pragma unroll
     for (int c = 0; c < NCG; ++c) st.bv[c] = colsum(st.bv[c]);
-    __syncthreads();   // slabs are dead from here on
-    float* sO = reinterpret_cast<float*>(lds_raw);
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) {
         const float bias = st.bv[ct / (GS / 16)];
@@ -477,6 +594,8 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
             st.o[ct][r] = v + partner(v);      // hi + lo
         }
     }
+    __syncthreads();   // slabs are dead from here on
+    float* sO = reinterpret_cast<float*>(lds_raw);
     if (col < g) {
 #pragma unroll
         for (int ct = 0; ct < 8; ++ct) {
@@ -488,6 +607,7 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
         }
     }
     __syncthreads();
+    const int64_t hstride = static_cast<int64_t>(P.b) * P.h;       // rows per split in the workspace
     for (int idx = tid; idx < g * kHeadDim; idx += kNW * 64) {
         const int hh = idx >> 7, c = idx & 127;
         float M = sM[0][hh];
@@ -510,35 +630,58 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
             P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(o);
             if (c == 0 && P.lse) P.lse[bi * P.h + hq] = empty ? INFINITY : lse;
         } else {
-            const int64_t row = (static_cast<int64_t>(split) * P.b + bi) * P.h + hq;
+            const int64_t row = split * hstride + bi * P.h + hq;
             P.o_part[row * kHeadDim + c] = o;
             if (c == 0) P.lse_part[row] = lse;
         }
     }
-}
+    if (P.nsplit == 1) return;
 
-// ---------------------------------------------------------------------------------------------
-// combine kernel: grid (b*h), 128 threads; follows flash_fwd_kernel.h:1217-1248, 1280-1298
-// ---------------------------------------------------------------------------------------------
-template <bool BF16>
-__global__ __launch_bounds__(128) void combine_kernel(FwdParams P) {
-    const int row = blockIdx.x;           // bi * h + hq
-    const int bi = row / P.h, hq = row % P.h;
-    const int c = threadIdx.x;
-    const int64_t stride = static_cast<int64_t>(P.b) * P.h;
-    float M = -INFINITY;
-    for (int s = 0; s < P.nsplit; ++s) M = fmaxf(M, P.lse_part[s * stride + row]);
-    const float Mu = (M == -INFINITY) ? 0.0f : M;
-    float sum = 0.0f;
-    for (int s = 0; s < P.nsplit; ++s) sum += __expf(P.lse_part[s * stride + row] - Mu);
-    const float L = (sum == 0.0f || sum != sum) ? INFINITY : __logf(sum) + Mu;
-    float o = 0.0f;
-    for (int s = 0; s < P.nsplit; ++s) {
-        const float w = __expf(P.lse_part[s * stride + row] - L);
-        o += w * P.o_part[(s * stride + row) * kHeadDim + c];
+    // ---- last workgroup of this (batch, kv-head) merges the splits.
+    // The barrier orders every thread's partial stores before thread 0's release increment at
+    // device scope; the workgroup that draws the last ticket acquires through the same atomic.
+    __syncthreads();
+    if (tid == 0) {
+        const int old = __hip_atomic_fetch_add(&P.tickets[bh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (old == P.nsplit - 1);
+        if (s_last) __hip_atomic_store(&P.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(o);
-    if (c == 0 && P.lse) P.lse[row] = L;
+    __syncthreads();
+    if (!s_last) return;
+    // split LSEs of the group's heads -> LDS, then every thread owns one (head, channel) and
+    // fetches its partial outputs sixteen at a time so that the loads overlap
+    float* sLse = reinterpret_cast<float*>(lds_raw);            // [split][g]
+    for (int idx = tid; idx < P.nsplit * g; idx += kNW * 64) {
+        const int sidx = idx / g, hh = idx - sidx * g;
+        sLse[idx] = P.lse_part[sidx * hstride + bi * P.h + hk * g + hh];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < g * kHeadDim; idx += kNW * 64) {
+        const int hh = idx >> 7, c = idx & 127;
+        const int hq = hk * g + hh;
+        const int64_t row0 = bi * P.h + hq;
+        float M = -INFINITY;
+        for (int sidx = 0; sidx < P.nsplit; ++sidx) M = fmaxf(M, sLse[sidx * g + hh]);
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        float sum = 0.0f, o = 0.0f;
+        for (int s0 = 0; s0 < P.nsplit; s0 += 16) {
+            float v[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                const int sidx = min(s0 + k, P.nsplit - 1);
+                v[k] = P.o_part[(sidx * hstride + row0) * kHeadDim + c];
+            }
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                const float w = (s0 + k < P.nsplit) ? __expf(sLse[(s0 + k) * g + hh] - Mu) : 0.0f;
+                sum += w;
+                o += w * v[k];
+            }
+        }
+        const bool none = (sum == 0.0f || sum != sum);
+        P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(none ? 0.0f : o / sum);
+        if (c == 0 && P.lse) P.lse[row0] = none ? INFINITY : __logf(sum) + Mu;
+    }
 }
 
 template <int BITS, int GS>
@@ -549,17 +692,7 @@ hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
     } else {
         hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, false>), grid, dim3(kNW * 64), 0, stream, P);
     }
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    if (P.nsplit > 1) {
-        if (P.bf16) {
-            hipLaunchKernelGGL((combine_kernel<true>), dim3(P.b * P.h), dim3(128), 0, stream, P);
-        } else {
-            hipLaunchKernelGGL((combine_kernel<false>), dim3(P.b * P.h), dim3(128), 0, stream, P);
-        }
-        e = hipGetLastError();
-    }
-    return e;
+    return hipGetLastError();
 }
 
 }  // namespace

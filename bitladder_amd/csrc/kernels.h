@@ -36,6 +36,7 @@ struct FwdParams {
     int seqlen, reslen;
     float* o_part;      // [split][b][h][128] normalised partial outputs
     float* lse_part;    // [split][b][h] natural-log LSE of each split
+    int* tickets;       // [b][h_k] arrival counters, zero between calls
     uint16_t* out;
     int64_t out_sb, out_sh;
     float* lse;         // optional [b][h]

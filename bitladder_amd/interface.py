@@ -270,7 +270,9 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
         a.num_splits = ns
         nbytes = L.bitdecode_fwd_workspace_bytes(b, h, ns)
         if nbytes:
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            # zero-filled: the arrival counters at its head must be 0 before the first call
+            # (every call leaves them at 0 again)
+            ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
             keep.append(ws)
             a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
     return DecodePlan(a, out, lse, tuple(keep), device)

@@ -80,7 +80,10 @@ typedef struct bitdecode_fwd_args {
     void* out;                 /* [b, 1, h, 128] element type of q                          */
     int64_t out_stride_b, out_stride_h;
     float* softmax_lse;        /* optional [b, h] natural-log LSE                           */
-    void* workspace;           /* >= bitdecode_fwd_workspace_bytes(...) or NULL if 1 split  */
+    void* workspace;           /* >= bitdecode_fwd_workspace_bytes(...) or NULL if 1 split;
+                                  its first 4*b*h bytes (arrival counters) must be zero before
+                                  the first call and are left zero by every call; calls that
+                                  share a workspace must not overlap in time                */
     size_t workspace_bytes;
     int32_t b, h, h_k, d;      /* d must be 128, h % h_k == 0, h / h_k <= 8                 */
     int32_t bits, group_size, dtype;
@@ -96,7 +99,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
 int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
                          int32_t num_cus);
 
-/* Workspace the split path needs: fp32 partial outputs and LSEs
+/* Workspace the split path needs: arrival counters, fp32 partial outputs and LSEs
  * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,
  * csrc/bit_decode/decode_api.cpp:292-295). */
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits);
