@@ -7,6 +7,7 @@
 #include <stdio.h>
 
 #include <algorithm>
+#include <cmath>
 
 #include "../../include/bitdecode.h"
 #include "kernels.h"
@@ -191,7 +192,8 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     P.lse = a->softmax_lse;
     P.b = a->b; P.h = a->h; P.hk = a->h_k; P.g = g; P.nsplit = nsplit;
     P.scale = a->softmax_scale;
-    P.scale_log2 = a->softmax_scale * 1.4426950408889634f;   // decode_api.cpp:128-142
+    P.scale_log2 = fabsf(a->softmax_scale) * 1.4426950408889634f;   // decode_api.cpp:128-142
+    P.neg_scale = a->softmax_scale < 0.0f;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
     if (nsplit > 1) {
         P.tickets = static_cast<int*>(a->workspace);
@@ -202,5 +204,9 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));
     return BITDECODE_OK;
 }
+
+#ifdef BITDECODE_PROF
+int bitdecode_prof_set(void* p) { return bitdecode::set_prof_buffer(static_cast<unsigned long long*>(p)) != hipSuccess; }
+#endif
 
 }  // extern "C"

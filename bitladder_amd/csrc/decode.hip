@@ -22,8 +22,12 @@
 //    an exact pair hi + lo (lo = fma(a, b, -hi)).  The 16 MFMA columns hold the GQA group twice:
 //    columns 0-7 carry the hi parts of heads 0-7, columns 8-15 the lo parts, so both go through
 //    the same MFMA and are added afterwards with one row-rotate (lane ^ 8) per accumulator.
-//  * Online softmax in base 2 per head (softmax.h:250-310), running max shared by the four
-//    lanes of a head through two cross-lane exchanges, row sums kept per lane until the end.
+//  * The offset/zero biases and the softmax row sums are themselves computed on the MFMA pipe
+//    (A operand = the zero vector / the constant offsets / ones), which keeps the VALU for the
+//    code unpacking; this kernel is VALU-issue bound long before it is MFMA bound.
+//  * Online softmax in base 2 per head (softmax.h:250-310) in steps of 32 tokens (64 at 2 bits):
+//    running max shared by the four lanes of a head through two lane-half swaps, accumulators
+//    rescaled only when some head's max actually moved.
 //  * The waves of a workgroup merge through LDS; splits merge in the same launch: the workgroup
 //    that draws the last ticket of a (batch, kv-head) combines all partials.
 #include <hip/hip_runtime.h>
@@ -40,6 +44,31 @@ typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+
+// Optional per-wave timeline for kernel tuning (built only with -DBITDECODE_PROF).
+#ifdef BITDECODE_PROF
+__device__ unsigned long long* g_prof = nullptr;
+#define PROF_DECL unsigned long long prof_ts[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define PROF(slot)                                 \
+    do {                                           \
+        __builtin_amdgcn_sched_barrier(0);         \
+        prof_ts[slot] = wall_clock64();            \
+        __builtin_amdgcn_sched_barrier(0);         \
+    } while (0)
+#define PROF_FLUSH()                                                                                  \
+    do {                                                                                              \
+        unsigned long long* pb = g_prof;                                                              \
+        if (pb && (threadIdx.x & 63) == 0) {                                                          \
+            pb += ((((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * kNW +   \
+                   (threadIdx.x >> 6)) * 8;                                                           \
+            for (int i_ = 0; i_ < 8; ++i_) pb[i_] = prof_ts[i_];                                      \
+        }                                                                                             \
+    } while (0)
+#else
+#define PROF_DECL do { } while (0)
+#define PROF(slot) do { } while (0)
+#define PROF_FLUSH() do { } while (0)
+#endif
 
 constexpr int kNW = 8;            // waves per workgroup
 constexpr float kPShift = 2.0f;   // probabilities are kept as 2^kPShift * exp2(s - max): a V scale
@@ -84,29 +113,39 @@ __device__ __forceinline__ float dot8(h8 a, h8 b, float c) {
     return c;
 }
 
+// The exponent patterns that turn a masked code field into offset + code (fp16).  They are kept
+// in VGPRs behind an empty asm so that (w & mask) | magic becomes one v_and_or_b32 (mask from an
+// SGPR, magic from a VGPR) instead of an AND and an OR with two literals.
+struct Magic {
+    uint32_t e1024, e256, e64, e16;
+    __device__ __forceinline__ Magic() : e1024(0x64006400u), e256(0x5c005c00u), e64(0x54005400u), e16(0x4c004c00u) {
+        asm volatile("" : "+v"(e1024), "+v"(e256), "+v"(e64), "+v"(e16));
+    }
+};
+
 // 8 four-bit codes -> (1024+c0, 1024+c4, 64+c1, 64+c5, 1024+c2, 1024+c6, 64+c3, 64+c7)
-__device__ __forceinline__ h8 dq4(uint32_t w) {
+__device__ __forceinline__ h8 dq4(uint32_t w, const Magic& mg) {
     u4 r;
-    r[0] = (w & 0x000f000fu) | 0x64006400u;
-    r[1] = (w & 0x00f000f0u) | 0x54005400u;
+    r[0] = (w & 0x000f000fu) | mg.e1024;
+    r[1] = (w & 0x00f000f0u) | mg.e64;
     const uint32_t w8 = w >> 8;
-    r[2] = (w8 & 0x000f000fu) | 0x64006400u;
-    r[3] = (w8 & 0x00f000f0u) | 0x54005400u;
+    r[2] = (w8 & 0x000f000fu) | mg.e1024;
+    r[3] = (w8 & 0x00f000f0u) | mg.e64;
     return __builtin_bit_cast(h8, r);
 }
 // 16 two-bit codes -> two k-steps; offsets per element (1024,1024,256,256,64,64,16,16)
-__device__ __forceinline__ void dq2(uint32_t w, h8& a0, h8& a1) {
+__device__ __forceinline__ void dq2(uint32_t w, h8& a0, h8& a1, const Magic& mg) {
     u4 r;
-    r[0] = (w & 0x00030003u) | 0x64006400u;
-    r[1] = (w & 0x000c000cu) | 0x5c005c00u;
-    r[2] = (w & 0x00300030u) | 0x54005400u;
-    r[3] = (w & 0x00c000c0u) | 0x4c004c00u;
+    r[0] = (w & 0x00030003u) | mg.e1024;
+    r[1] = (w & 0x000c000cu) | mg.e256;
+    r[2] = (w & 0x00300030u) | mg.e64;
+    r[3] = (w & 0x00c000c0u) | mg.e16;
     a0 = __builtin_bit_cast(h8, r);
     const uint32_t w8 = w >> 8;
-    r[0] = (w8 & 0x00030003u) | 0x64006400u;
-    r[1] = (w8 & 0x000c000cu) | 0x5c005c00u;
-    r[2] = (w8 & 0x00300030u) | 0x54005400u;
-    r[3] = (w8 & 0x00c000c0u) | 0x4c004c00u;
+    r[0] = (w8 & 0x00030003u) | mg.e1024;
+    r[1] = (w8 & 0x000c000cu) | mg.e256;
+    r[2] = (w8 & 0x00300030u) | mg.e64;
+    r[3] = (w8 & 0x00c000c0u) | mg.e16;
     a1 = __builtin_bit_cast(h8, r);
 }
 
@@ -137,44 +176,47 @@ __device__ __forceinline__ h8 split_mul(h8 a, h8 b, bool lo_part) {
     return lo_part ? lo : hi;
 }
 
-// sum / max over the four lanes that share a column (lane, lane^16, lane^32, lane^48)
-__device__ __forceinline__ float colsum(float x) {
-    x += __shfl_xor(x, 16);
-    x += __shfl_xor(x, 32);
-    return x;
-}
+// max over the four lanes that share a column (lane, lane^16, lane^32, lane^48)
 __device__ __forceinline__ float colmax(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16));
-    x = fmaxf(x, __shfl_xor(x, 32));
-    return x;
+    unsigned u = __builtin_bit_cast(unsigned, x);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);   // rows (0,0,2,2) and (1,1,3,3)
+    x = fmaxf(__builtin_bit_cast(float, a[0]), __builtin_bit_cast(float, a[1]));
+    u = __builtin_bit_cast(unsigned, x);
+    auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // halves (lo,lo) and (hi,hi)
+    return fmaxf(__builtin_bit_cast(float, b[0]), __builtin_bit_cast(float, b[1]));
 }
 
 template <int NCG>
 struct WaveState {
-    float m;          // running max of the base-2 scores of this lane's head
-    float l;          // this lane's share of sum p
-    float bv[NCG];    // this lane's share of the V bias per channel group
+    float m;          // running max of the raw scores (q.k units) of this lane's head
+    f4 l;             // sum of p, accumulated by MFMA against a ones operand (hi columns only)
+    f4 ob[NCG];       // V bias per channel group, accumulated by MFMA (all four rows equal)
     f4 o[8];          // O^T tiles: lane (head, q) holds channels 16*ct + 4*q + r
 };
 
-// Online-softmax step over N scores; returns p = 2^kPShift * exp2(s - max) in place.
+// Online-softmax step over N raw scores t (q.k units); on return t holds
+// p = 2^kPShift * exp2(scale * (t - running max)).  Accumulators are rescaled only when the
+// running max of some head moved (wave-uniform branch).
 template <int N, int NCG>
-__device__ __forceinline__ void softmax_step(float (&s)[N], WaveState<NCG>& st) {
-    float mx = s[0];
+__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st) {
+    float mx = t[0];
 #pragma unroll
-    for (int i = 1; i < N; ++i) mx = fmaxf(mx, s[i]);
+    for (int i = 1; i < N; ++i) mx = fmaxf(mx, t[i]);
     mx = colmax(mx);
     const float m_new = fmaxf(st.m, mx);
     const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);
+    if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
+        const float alpha = __builtin_amdgcn_exp2f((st.m - m_use) * scale);
+        st.l *= alpha;
 #pragma unroll
-    for (int i = 0; i < N; ++i) s[i] = __builtin_amdgcn_exp2f(s[i] - m_use + kPShift);
-    st.l *= alpha;
+        for (int c = 0; c < NCG; ++c) st.ob[c] *= alpha;
 #pragma unroll
-    for (int c = 0; c < NCG; ++c) st.bv[c] *= alpha;
+        for (int ct = 0; ct < 8; ++ct) st.o[ct] *= alpha;
+        st.m = m_new;
+    }
+    const float c0 = kPShift - m_use * scale;
 #pragma unroll
-    for (int ct = 0; ct < 8; ++ct) st.o[ct] *= alpha;
-    st.m = m_new;
+    for (int i = 0; i < N; ++i) t[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(t[i], scale, c0));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -206,16 +248,17 @@ __device__ __forceinline__ void load_kside(KSide<BITS, GS>& K, const FwdParams& 
     const int kg = lane >> 4;
     const uint8_t* kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
     const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
+    const uint32_t poff = kg * 16, coff = lane * 16;     // per-lane byte offsets from uniform bases
 #pragma unroll
     for (int g = 0; g < KSide<BITS, GS>::PF; ++g) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            K.ps[g][j] = ld_u4(kp + g * kKParamGroupBytes + (32 * j + 8 * kg) * 2);
-            K.pz[g][j] = ld_u4(kp + g * kKParamGroupBytes + 256 + (32 * j + 8 * kg) * 2);
+            K.ps[g][j] = ld_u4(kp + (g * kKParamGroupBytes + 64 * j) + poff);
+            K.pz[g][j] = ld_u4(kp + (g * kKParamGroupBytes + 256 + 64 * j) + poff);
         }
     }
 #pragma unroll
-    for (int x = 0; x < KSide<BITS, GS>::NW4; ++x) K.code[x] = ld_u4(kc + x * 1024 + lane * 16);
+    for (int x = 0; x < KSide<BITS, GS>::NW4; ++x) K.code[x] = ld_u4(kc + x * 1024 + coff);
 }
 
 template <int BITS, int GS>
@@ -223,171 +266,132 @@ __device__ __forceinline__ void load_vside(VSide<BITS, GS>& V, const FwdParams& 
     const int kg = lane >> 4;
     const uint8_t* vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
     const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
+    const uint32_t poff = kg * 16, coff = lane * 16;
 #pragma unroll
     for (int sb = 0; sb < VSide<BITS, GS>::PF; ++sb) {
-        V.ps[sb] = ld_u4(vp + sb * 128 + kg * 16);
-        V.pz[sb] = ld_u4(vp + sb * 128 + 64 + kg * 16);
+        V.ps[sb] = ld_u4(vp + sb * 128 + poff);
+        V.pz[sb] = ld_u4(vp + (sb * 128 + 64) + poff);
     }
 #pragma unroll
-    for (int x = 0; x < VSide<BITS, GS>::NW4; ++x) V.code[x] = ld_u4(vc + x * 1024 + lane * 16);
+    for (int x = 0; x < VSide<BITS, GS>::NW4; ++x) V.code[x] = ld_u4(vc + x * 1024 + coff);
 }
 
-// S^T = K Q^T for the 8 tiles of a chunk, then the online-softmax step.  On return s[] holds
-// the probabilities 2^kPShift * exp2(score - running max) of this lane's 32 tokens.
+// One packed chunk in steps of 32 tokens (4-bit) or 64 tokens (2-bit): S^T tiles of the step,
+// online-softmax update, O^T += V^T P^T for the same tokens.  Scores stay in q.k units; the
+// softmax scale is applied inside the exponent.
 template <int BITS, int GS, bool BF16>
-__device__ __forceinline__ void chunk_scores(const KSide<BITS, GS>& K, const FwdParams& P, int64_t bh, int ci,
-                                             int lane, const h8 (&qB)[4], bool lo_part, float (&s)[32],
-                                             WaveState<kHeadDim / GS>& st) {
+__device__ __forceinline__ void packed_chunk(const KSide<BITS, GS>& K, const VSide<BITS, GS>& V, const FwdParams& P,
+                                             int64_t bh, int ci, int lane, const h8 (&qB)[4], bool lo_part,
+                                             const Magic& mg, WaveState<kHeadDim / GS>& st) {
     constexpr int NG = kChunk / GS;
     constexpr int NCG = kHeadDim / GS;
-    constexpr int TPG = GS / 16;      // 16-token tiles per K group
-    constexpr int PF = KSide<BITS, GS>::PF;
+    constexpr int TPG = GS / 16;                 // 16-token tiles per K group
+    constexpr int CTPG = GS / 16;                // 16-channel tiles per V channel group
+    constexpr int TPS = BITS == 4 ? 2 : 4;       // tiles per step
+    constexpr int NSTEP = 8 / TPS;
+    constexpr int KPF = KSide<BITS, GS>::PF;
+    constexpr int VPF = VSide<BITS, GS>::PF;
     const int kg = lane >> 4;
-    const h8 off = code_offsets<BITS>();
-    const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
-
-#pragma unroll
-    for (int grp = 0; grp < NG; ++grp) {
-        h8 qp[4];
-        float kap = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            u4 rs, rz;
-            if (grp < PF) {
-                rs = K.ps[grp < PF ? grp : 0][j];
-                rz = K.pz[grp < PF ? grp : 0][j];
-            } else {
-                rs = ld_u4(kp + grp * kKParamGroupBytes + (32 * j + 8 * kg) * 2);
-                rz = ld_u4(kp + grp * kKParamGroupBytes + 256 + (32 * j + 8 * kg) * 2);
-            }
-            const h8 sc = cvt_h8<BF16>(rs), zr = cvt_h8<BF16>(rz);
-            qp[j] = split_mul(qB[j], sc, lo_part);
-            if (!lo_part) kap = dot8(qB[j], zr, kap);
-            kap = -dot8(qp[j], off, -kap);
-        }
-        kap = colsum(kap) * P.scale_log2;
-        if constexpr (BITS == 4) {
-#pragma unroll
-            for (int tt = 0; tt < TPG; ++tt) {
-                const int t = grp * TPG + tt;
-                const u4 w = K.code[t];
-                f4 acc = {0, 0, 0, 0};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc = mfma32(dq4(w[j]), qp[j], acc);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float sp = acc[r] * P.scale_log2 + kap;
-                    s[4 * t + r] = sp + partner(sp);
-                }
-            }
-        } else {
-#pragma unroll
-            for (int pp = 0; pp < TPG / 2; ++pp) {
-                const int tp = grp * (TPG / 2) + pp;
-                const u4 w = K.code[tp];
-#pragma unroll
-                for (int tin = 0; tin < 2; ++tin) {
-                    f4 acc = {0, 0, 0, 0};
-#pragma unroll
-                    for (int jj = 0; jj < 2; ++jj) {
-                        h8 a0, a1;
-                        dq2(w[2 * tin + jj], a0, a1);
-                        acc = mfma32(a0, qp[2 * jj], acc);
-                        acc = mfma32(a1, qp[2 * jj + 1], acc);
-                    }
-                    const int t = 2 * tp + tin;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float sp = acc[r] * P.scale_log2 + kap;
-                        s[4 * t + r] = sp + partner(sp);
-                    }
-                }
-            }
-        }
-    }
-    softmax_step<32, NCG>(s, st);
-}
-
-// O^T += V^T P^T for one chunk, 32 tokens (one k-step) at a time
-template <int BITS, int GS, bool BF16>
-__device__ __forceinline__ void chunk_pv(const VSide<BITS, GS>& V, const FwdParams& P, int64_t bh, int ci, int lane,
-                                         bool lo_part, const float (&s)[32], WaveState<kHeadDim / GS>& st) {
-    constexpr int NCG = kHeadDim / GS;
-    constexpr int CTPG = GS / 16;     // 16-channel tiles per V channel group
-    constexpr int PF = VSide<BITS, GS>::PF;
-    const int kg = lane >> 4;
-    const h8 off = code_offsets<BITS>();
+    const h8 noff = -code_offsets<BITS>();
     const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
+    const h8 zero8 = h8{0, 0, 0, 0, 0, 0, 0, 0};
+    const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
     const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
 
-    h8 p16[4];
+    h8 qp[4];
+    f4 kb = {0, 0, 0, 0};
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb) {
+    for (int step = 0; step < NSTEP; ++step) {
+        float t[4 * TPS];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            // element i = 4*T + r  <->  tile 2*sb + T, accumulator register r
-            const int i0 = 2 * x;
-            const int t0 = 2 * sb + i0 / 4, r0 = i0 % 4;
-            h2 t = pk_rtz(s[4 * t0 + r0], s[4 * t0 + r0 + 1]);
-            p16[sb][2 * x] = t[0];
-            p16[sb][2 * x + 1] = t[1];
-        }
-        st.l = dot8(p16[sb], ones, st.l);
-    }
-
-    auto params = [&](int sb, int cg, h8& vs, h8& vz) {
-        if (PF) {
-            vs = cvt_h8<BF16>(V.ps[PF ? sb : 0]);
-            vz = cvt_h8<BF16>(V.pz[PF ? sb : 0]);
-        } else {
-            vs = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + kg * 16);
-            vz = ld_h8<BF16>(vp + (sb * NCG + cg) * 128 + 64 + kg * 16);
-        }
-    };
-
-    if constexpr (BITS == 4) {
+        for (int tt = 0; tt < TPS; ++tt) {
+            const int tile = step * TPS + tt;
+            if (tile % TPG == 0) {
+                // new K group: fold its scale into Q (exact hi/lo split) and build the score bias
+                // sum_c q_c*zero_c - sum_c (q_c*scale_c)*offset_c on the MFMA pipe
+                const int grp = tile / TPG;
+                kb = f4{0, 0, 0, 0};
 #pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {
-            const u4 w0 = V.code[2 * sb], w1 = V.code[2 * sb + 1];
-#pragma unroll
-            for (int cg = 0; cg < NCG; ++cg) {
-                h8 vs, vz;
-                params(sb, cg, vs, vz);
-                const h8 pp = split_mul(p16[sb], vs, lo_part);
-                if (!lo_part) st.bv[cg] = dot8(p16[sb], vz, st.bv[cg]);
-                st.bv[cg] = -dot8(pp, off, -st.bv[cg]);
-#pragma unroll
-                for (int x = 0; x < CTPG; ++x) {
-                    const int ct = cg * CTPG + x;
-                    const uint32_t w = ct < 4 ? w0[ct & 3] : w1[ct & 3];
-                    st.o[ct] = mfma32(dq4(w), pp, st.o[ct]);
+                for (int j = 0; j < 4; ++j) {
+                    u4 rs, rz;
+                    if (grp < KPF) {
+                        rs = K.ps[grp < KPF ? grp : 0][j];
+                        rz = K.pz[grp < KPF ? grp : 0][j];
+                    } else {
+                        rs = ld_u4(kp + (grp * kKParamGroupBytes + 64 * j) + kg * 16);
+                        rz = ld_u4(kp + (grp * kKParamGroupBytes + 256 + 64 * j) + kg * 16);
+                    }
+                    qp[j] = split_mul(qB[j], cvt_h8<BF16>(rs), lo_part);
+                    kb = mfma32(cvt_h8<BF16>(rz), lo_part ? zero8 : qB[j], kb);
+                    kb = mfma32(noff, qp[j], kb);
                 }
             }
-        }
-    } else {
+            f4 acc = kb;
+            if constexpr (BITS == 4) {
+                const u4 w = K.code[tile];
 #pragma unroll
-        for (int sb2 = 0; sb2 < 2; ++sb2) {
-            const u4 w0 = V.code[2 * sb2], w1 = V.code[2 * sb2 + 1];
+                for (int j = 0; j < 4; ++j) acc = mfma32(dq4(w[j], mg), qp[j], acc);
+            } else {
+                const u4 w = K.code[tile / 2];
 #pragma unroll
-            for (int cg = 0; cg < NCG; ++cg) {
-                h8 pp[2];
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const int sb = 2 * sb2 + ks;
-                    h8 vs, vz;
-                    params(sb, cg, vs, vz);
-                    pp[ks] = split_mul(p16[sb], vs, lo_part);
-                    if (!lo_part) st.bv[cg] = dot8(p16[sb], vz, st.bv[cg]);
-                    st.bv[cg] = -dot8(pp[ks], off, -st.bv[cg]);
-                }
-#pragma unroll
-                for (int x = 0; x < CTPG; ++x) {
-                    const int ct = cg * CTPG + x;
-                    const uint32_t w = ct < 4 ? w0[ct & 3] : w1[ct & 3];
+                for (int jj = 0; jj < 2; ++jj) {
                     h8 a0, a1;
-                    dq2(w, a0, a1);
+                    dq2(w[2 * (tile % 2) + jj], a0, a1, mg);
+                    acc = mfma32(a0, qp[2 * jj], acc);
+                    acc = mfma32(a1, qp[2 * jj + 1], acc);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) t[4 * tt + r] = acc[r] + partner(acc[r]);   // hi + lo
+        }
+
+        softmax_step<4 * TPS, NCG>(t, P.scale_log2, st);
+
+        // ---- O^T += V^T P^T for the tokens of this step
+        constexpr int NKS = TPS / 2;                  // 32-token k-steps in this step
+        h8 p16[NKS], pz[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                // element i = 4*T + r  <->  tile 2*ks + T of the step, accumulator register r
+                const h2 pr = pk_rtz(t[8 * ks + 2 * x], t[8 * ks + 2 * x + 1]);
+                p16[ks][2 * x] = pr[0];
+                p16[ks][2 * x + 1] = pr[1];
+            }
+            pz[ks] = lo_part ? zero8 : p16[ks];       // p itself only in the hi columns
+            st.l = mfma32(ones, pz[ks], st.l);
+        }
+        const u4 w0 = V.code[2 * step], w1 = V.code[2 * step + 1];
+#pragma unroll
+        for (int cg = 0; cg < NCG; ++cg) {
+            h8 pp[NKS];
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int sb = step * NKS + ks;
+                u4 rs, rz;
+                if (VPF) {
+                    rs = V.ps[VPF ? sb : 0];
+                    rz = V.pz[VPF ? sb : 0];
+                } else {
+                    rs = ld_u4(vp + (sb * NCG + cg) * 128 + kg * 16);
+                    rz = ld_u4(vp + ((sb * NCG + cg) * 128 + 64) + kg * 16);
+                }
+                pp[ks] = split_mul(p16[ks], cvt_h8<BF16>(rs), lo_part);
+                st.ob[cg] = mfma32(cvt_h8<BF16>(rz), pz[ks], st.ob[cg]);
+                st.ob[cg] = mfma32(noff, pp[ks], st.ob[cg]);
+            }
+#pragma unroll
+            for (int x = 0; x < CTPG; ++x) {
+                const int ct = cg * CTPG + x;
+                const uint32_t w = ct < 4 ? w0[ct & 3] : w1[ct & 3];
+                if constexpr (BITS == 4) {
+                    st.o[ct] = mfma32(dq4(w, mg), pp[0], st.o[ct]);
+                } else {
+                    h8 a0, a1;
+                    dq2(w, a0, a1, mg);
                     st.o[ct] = mfma32(a0, pp[0], st.o[ct]);
-                    st.o[ct] = mfma32(a1, pp[1], st.o[ct]);
+                    st.o[ct] = mfma32(a1, pp[NKS - 1], st.o[ct]);
                 }
             }
         }
@@ -447,17 +451,15 @@ __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P,
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int tk = n0 + 4 * kg + r;
-            const float sp = acc[r] * P.scale_log2;
-            const float tot = sp + partner(sp);     // outside the select: every lane must execute the DPP
+            const float tot = acc[r] + partner(acc[r]);   // outside the select: every lane executes the DPP
             s[r] = tk < R ? tot : -INFINITY;
         }
     }
-    softmax_step<4, NCG>(s, st);
+    softmax_step<4, NCG>(s, P.scale_log2, st);
     const h2 p01 = pk_rtz(s[0], s[1]), p23 = pk_rtz(s[2], s[3]);
-    st.l = __builtin_amdgcn_fdot2(p01, h2{1, 1}, st.l, false);
-    st.l = __builtin_amdgcn_fdot2(p23, h2{1, 1}, st.l, false);
     h4 pb = {p01[0], p01[1], p23[0], p23[1]};
     if (lo_part) pb = h4{0, 0, 0, 0};
+    st.l = mfma16(h4{1, 1, 1, 1}, pb, st.l);
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) {
         uint16_t e[4];
@@ -476,6 +478,14 @@ __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P,
         }
         st.o[ct] = mfma16(a, pb, st.o[ct]);
     }
+}
+
+// device-scope (agent) relaxed accesses: write-through stores / cache-coherent loads
+__device__ __forceinline__ void st_dev(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_dev(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <bool BF16>
@@ -508,8 +518,11 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
     __shared__ float sM[kNW][kMaxGroupHeads], sL[kNW][kMaxGroupHeads];
     __shared__ int s_last;
 
+    PROF_DECL;
+    PROF(0);
     const int split = blockIdx.x, hk = blockIdx.y, bi = blockIdx.z;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: chunk addresses stay in SGPRs
     const int col = lane & 15, kg = lane >> 4;
     const int head = col & 7;          // query head inside the GQA group
     const bool lo_part = col >= 8;     // columns 8-15 carry the lo halves of the split products
@@ -524,38 +537,57 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
     const int c1 = min(nP, c0 + cps);
     const int nT = (R + 15) / 16;
 
-    h8 qB[4];
+    // Q is fetched unconditionally (padding columns re-read head 0 and are zeroed after the
+    // chunk loads have been issued) so that no wait sits in front of the big loads.
+    u4 qraw[4];
+    {
+        const uint16_t* qp = P.q + bi * P.q_sb + (hk * g + (head < g ? head : 0)) * P.q_sh + 8 * kg;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        qB[j] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (head < g) qB[j] = ld_h8<BF16>(P.q + bi * P.q_sb + (hk * g + head) * P.q_sh + 32 * j + 8 * kg);
+        for (int j = 0; j < 4; ++j) qraw[j] = ld_u4(qp + 32 * j);
     }
+    auto q_operand = [&](h8 (&qB)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (head >= g) qraw[j] = u4{0, 0, 0, 0};
+            qB[j] = cvt_h8<BF16>(qraw[j]);
+            if (P.neg_scale) qB[j] = -qB[j];     // scale_log2 holds |scale|: running max needs scale >= 0
+        }
+    };
 
     WaveState<NCG> st;
     st.m = -INFINITY;
-    st.l = 0.0f;
+    st.l = f4{0, 0, 0, 0};
 #pragma unroll
-    for (int c = 0; c < NCG; ++c) st.bv[c] = 0.0f;
+    for (int c = 0; c < NCG; ++c) st.ob[c] = f4{0, 0, 0, 0};
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) st.o[ct] = f4{0, 0, 0, 0};
 
     // ---- packed chunks of this wave, software-pipelined one side ahead
+    h8 qB[4];
     {
         int ci = c0 + wave;
-        if (ci < c1) {
+        if (ci >= c1) {
+            q_operand(qB);
+        } else {
             KSide<BITS, GS> K;
             VSide<BITS, GS> V;
+            const Magic mg;
+            PROF(1);
             load_kside<BITS, GS>(K, P, bh, ci, lane);
             load_vside<BITS, GS>(V, P, bh, ci, lane);
+            // every load of the chunk is issued before any of it is used: keep the scheduler from
+            // sinking the V loads below the QK^T work
+            __builtin_amdgcn_sched_barrier(0);
+            PROF(2);
+            q_operand(qB);
             while (true) {
-                float s[32];
-                chunk_scores<BITS, GS, BF16>(K, P, bh, ci, lane, qB, lo_part, s, st);
+                packed_chunk<BITS, GS, BF16>(K, V, P, bh, ci, lane, qB, lo_part, mg, st);
+                PROF(3);
                 const int cn = ci + kNW;
-                const bool more = cn < c1;
-                if (more) load_kside<BITS, GS>(K, P, bh, cn, lane);
-                chunk_pv<BITS, GS, BF16>(V, P, bh, ci, lane, lo_part, s, st);
-                if (!more) break;
+                if (cn >= c1) break;
+                load_kside<BITS, GS>(K, P, bh, cn, lane);
                 load_vside<BITS, GS>(V, P, bh, cn, lane);
+                __builtin_amdgcn_sched_barrier(0);
                 ci = cn;
             }
         }
@@ -581,16 +613,14 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
         }
     }
 
+    PROF(4);
     // ---- merge the waves of this workgroup through LDS
-    st.l = colsum(st.l);
-#pragma unroll
-    for (int c = 0; c < NCG; ++c) st.bv[c] = colsum(st.bv[c]);
+    const float lsum = st.l[0] + partner(st.l[0]);      // rows are equal; lo columns hold 0
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) {
-        const float bias = st.bv[ct / (GS / 16)];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float v = st.o[ct][r] + bias;
+            const float v = st.o[ct][r] + st.ob[ct / (GS / 16)][r];
             st.o[ct][r] = v + partner(v);      // hi + lo
         }
     }
@@ -602,8 +632,8 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
             *reinterpret_cast<f4*>(&sO[(wave * kMaxGroupHeads + col) * kHeadDim + 16 * ct + 4 * kg]) = st.o[ct];
         }
         if (kg == 0) {
-            sM[wave][col] = st.m;
-            sL[wave][col] = st.l;
+            sM[wave][col] = st.m * P.scale_log2;     // base-2 units
+            sL[wave][col] = lsum;
         }
     }
     __syncthreads();
@@ -631,57 +661,74 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
             if (c == 0 && P.lse) P.lse[bi * P.h + hq] = empty ? INFINITY : lse;
         } else {
             const int64_t row = split * hstride + bi * P.h + hq;
-            P.o_part[row * kHeadDim + c] = o;
-            if (c == 0) P.lse_part[row] = lse;
+            st_dev(&P.o_part[row * kHeadDim + c], o);
+            if (c == 0) st_dev(&P.lse_part[row], lse);
         }
     }
-    if (P.nsplit == 1) return;
+    PROF(5);
+    if (P.nsplit == 1) {
+        PROF_FLUSH();
+        return;
+    }
 
-    // ---- last workgroup of this (batch, kv-head) merges the splits.
-    // The barrier orders every thread's partial stores before thread 0's release increment at
-    // device scope; the workgroup that draws the last ticket acquires through the same atomic.
+    // ---- the workgroup that draws the last ticket of this (batch, kv-head) merges the splits.
+    // Partials are written with device-scope (write-through) stores; once a thread's stores have
+    // completed (vmcnt 0) and the workgroup has met at the barrier, thread 0 takes the ticket.
+    // The merging workgroup reads the partials with device-scope loads, so no cache-wide
+    // write-back or invalidate is needed on either side.
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this thread's partial stores are complete
     __syncthreads();
     if (tid == 0) {
-        const int old = __hip_atomic_fetch_add(&P.tickets[bh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = __hip_atomic_fetch_add(&P.tickets[bh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (old == P.nsplit - 1);
         if (s_last) __hip_atomic_store(&P.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    if (!s_last) return;
-    // split LSEs of the group's heads -> LDS, then every thread owns one (head, channel) and
-    // fetches its partial outputs sixteen at a time so that the loads overlap
-    float* sLse = reinterpret_cast<float*>(lds_raw);            // [split][g]
-    for (int idx = tid; idx < P.nsplit * g; idx += kNW * 64) {
-        const int sidx = idx / g, hh = idx - sidx * g;
-        sLse[idx] = P.lse_part[sidx * hstride + bi * P.h + hk * g + hh];
+    PROF(6);
+    if (!s_last) {
+        PROF_FLUSH();
+        return;
     }
-    __syncthreads();
+    // every thread owns one (head, channel) and fetches the partial outputs and LSEs of up to 32
+    // splits in one batch, so that the whole merge costs one memory round trip
     for (int idx = tid; idx < g * kHeadDim; idx += kNW * 64) {
         const int hh = idx >> 7, c = idx & 127;
         const int hq = hk * g + hh;
         const int64_t row0 = bi * P.h + hq;
-        float M = -INFINITY;
-        for (int sidx = 0; sidx < P.nsplit; ++sidx) M = fmaxf(M, sLse[sidx * g + hh]);
-        const float Mu = (M == -INFINITY) ? 0.0f : M;
-        float sum = 0.0f, o = 0.0f;
-        for (int s0 = 0; s0 < P.nsplit; s0 += 16) {
-            float v[16];
+        float M = -INFINITY, sum = 0.0f, o = 0.0f;
+        for (int s0 = 0; s0 < P.nsplit; s0 += 32) {
+            float v[32], e[32];
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
+            for (int k = 0; k < 32; ++k) {
                 const int sidx = min(s0 + k, P.nsplit - 1);
-                v[k] = P.o_part[(sidx * hstride + row0) * kHeadDim + c];
+                v[k] = ld_dev(&P.o_part[(sidx * hstride + row0) * kHeadDim + c]);
+                e[k] = ld_dev(&P.lse_part[sidx * hstride + row0]);
             }
+            float mb = -INFINITY;
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
-                const float w = (s0 + k < P.nsplit) ? __expf(sLse[(s0 + k) * g + hh] - Mu) : 0.0f;
+            for (int k = 0; k < 32; ++k) {
+                if (s0 + k >= P.nsplit) e[k] = -INFINITY;
+                mb = fmaxf(mb, e[k]);
+            }
+            const float Mn = fmaxf(M, mb);
+            const float Mu = (Mn == -INFINITY) ? 0.0f : Mn;
+            const float a = __expf(M - Mu);
+            sum *= a;
+            o *= a;
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                const float w = __expf(e[k] - Mu);
                 sum += w;
                 o += w * v[k];
             }
+            M = Mn;
         }
         const bool none = (sum == 0.0f || sum != sum);
         P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(none ? 0.0f : o / sum);
-        if (c == 0 && P.lse) P.lse[row0] = none ? INFINITY : __logf(sum) + Mu;
+        if (c == 0 && P.lse) P.lse[row0] = none ? INFINITY : __logf(sum) + M;
     }
+    PROF(7);
+    PROF_FLUSH();
 }
 
 template <int BITS, int GS>
@@ -696,6 +743,12 @@ hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
 }
 
 }  // namespace
+
+#ifdef BITDECODE_PROF
+hipError_t set_prof_buffer(unsigned long long* p) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_prof), &p, sizeof(p));
+}
+#endif
 
 hipError_t launch_fwd(const FwdParams& P, hipStream_t stream) {
     switch (P.bits * 1000 + P.gs) {

@@ -41,11 +41,15 @@ struct FwdParams {
     int64_t out_sb, out_sh;
     float* lse;         // optional [b][h]
     int b, h, hk, g, nsplit;
-    float scale, scale_log2;
+    float scale, scale_log2;   // scale_log2 = |softmax_scale| * log2(e)
+    int neg_scale;             // softmax_scale < 0: the sign is folded into q
     int bits, gs, bf16;
 };
 
 hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);
 hipError_t launch_fwd(const FwdParams& p, hipStream_t stream);
+#ifdef BITDECODE_PROF
+hipError_t set_prof_buffer(unsigned long long* p);   // per-wave timeline buffer (tuning builds only)
+#endif
 
 }  // namespace bitdecode
