@@ -176,14 +176,19 @@ __device__ __forceinline__ h8 split_mul(h8 a, h8 b, bool lo_part) {
     return lo_part ? lo : hi;
 }
 
-// max over the four lanes that share a column (lane, lane^16, lane^32, lane^48)
+// max over the four lanes that share a column (lane, lane^16, lane^32, lane^48).
+// v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of
+// its second one, v_permlane32_swap does the same with 32-lane halves; fed two copies of x they
+// leave (rows 0,0,2,2 / rows 1,1,3,3) and (lower,lower / upper,upper), whose element-wise max is
+// the reduction.  Written as asm: the compiler builtin folds the two results into one here.
+// The s_nop covers the wait states the swap needs after a VALU write of its operands.
 __device__ __forceinline__ float colmax(float x) {
-    unsigned u = __builtin_bit_cast(unsigned, x);
-    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);   // rows (0,0,2,2) and (1,1,3,3)
-    x = fmaxf(__builtin_bit_cast(float, a[0]), __builtin_bit_cast(float, a[1]));
-    u = __builtin_bit_cast(unsigned, x);
-    auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // halves (lo,lo) and (hi,hi)
-    return fmaxf(__builtin_bit_cast(float, b[0]), __builtin_bit_cast(float, b[1]));
+    float y = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    x = fmaxf(x, y);
+    y = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    return fmaxf(x, y);
 }
 
 template <int NCG>

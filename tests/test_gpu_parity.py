@@ -100,3 +100,20 @@ def test_decode_residual_only(device):
                               v_residual=H.to_dev(v, "fp16", device), num_splits=ns)
         err = np.abs(out.float().cpu().numpy() - want).max()
         assert err < ATOL, (ns, err)
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 128), (4, 64), (4, 32), (2, 128), (2, 64), (2, 32)])
+def test_decode_many_chunks_per_wave(device, bits, gs):
+    """Few splits over a long prefix: every wave loops over several chunks (running max carried
+    across chunks, loads of the next chunk issued while the current one is consumed)."""
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, S = 1, 8, 2, 4096 + 128 * 3          # 35 chunks: uneven tail across the 8 waves
+    q, k, v = O.make_inputs(b, h, h_k, S, 0, seed=21)
+    qkv = O.quantize_kv_ref(k, v, bits, gs)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, _ = O.attend_ref(q, k_hat, v_hat, SCALE)
+    for ns in (1, 2):
+        out = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns)
+        err = np.abs(out.float().cpu().numpy() - want).max()
+        assert err < ATOL, (ns, err)

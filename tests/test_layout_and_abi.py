@@ -1,0 +1,226 @@
+"""CPU tests: physical layout description, C-ABI exports and host-side argument checks.
+No GPU compute is issued: every C-ABI call made here fails validation before any launch."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from bitladder_amd import _lib
+from bitladder_amd import layout as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_layout_roundtrip_and_byte_budget(bits, gs):
+    rng = np.random.default_rng(bits * 1000 + gs)
+    b, S, h = 2, 256, 3
+    kc = rng.integers(0, 1 << bits, (b, S, h, 128), dtype=np.uint8)
+    vc = rng.integers(0, 1 << bits, (b, S, h, 128), dtype=np.uint8)
+    ks = rng.integers(0, 65536, (b, S // gs, h, 128)).astype(np.uint16)
+    kz = rng.integers(0, 65536, (b, S // gs, h, 128)).astype(np.uint16)
+    vs = rng.integers(0, 65536, (b, S, h, 128 // gs)).astype(np.uint16)
+    vz = rng.integers(0, 65536, (b, S, h, 128 // gs)).astype(np.uint16)
+    phys = L.pack_physical(kc, ks, kz, vc, vs, vz, bits, gs)
+    pn = 16 // bits
+    # the reference's tensor contract (evaluation/test.py:76-83)
+    assert phys[0].shape == (b, S // pn, h, 128) and phys[0].dtype == np.uint16
+    assert phys[1].shape == (b, S // gs, h, 128) and phys[1].dtype == np.float32
+    assert phys[2].shape == (b, S, h, 128 // pn) and phys[2].dtype == np.uint16
+    assert phys[3].shape == (b, 128 // gs, h, S) and phys[3].dtype == np.float32
+    back = L.unpack_physical(*phys, bits, gs)
+    for a, c in zip((kc, ks, kz, vc, vs, vz), back):
+        np.testing.assert_array_equal(a, c)
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_code_maps_are_bijections_and_chunk_local(bits):
+    for fn in (L.k_code_map, L.v_code_map):
+        tok, ch = fn(bits)
+        assert tok.shape == (128 * 128 * bits // 32, 32 // bits)
+        pairs = set(zip(tok.ravel().tolist(), ch.ravel().tolist()))
+        assert len(pairs) == 128 * 128
+        assert tok.min() == 0 and tok.max() == 127 and ch.min() == 0 and ch.max() == 127
+
+
+def test_k_dword_holds_one_token_and_v_dword_one_channel():
+    """A K dword feeds the MFMA A operand of S^T = K Q^T (8 channels of one token); a V dword
+    feeds the A operand of O^T = V^T P^T (8 tokens of one channel)."""
+    for bits in (2, 4):
+        tok, ch = L.k_code_map(bits)
+        assert (tok == tok[:, :1]).all()
+        tok, ch = L.v_code_map(bits)
+        assert (ch == ch[:, :1]).all()
+
+
+def test_chunks_are_independent_regions():
+    """Packing two chunks at once equals packing them separately and concatenating per head:
+    what lets 128 new tokens be appended without touching the rest of the cache."""
+    rng = np.random.default_rng(3)
+    bits, gs, b, h = 4, 128, 1, 2
+    mk = lambda S: (rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8),
+                    rng.integers(0, 65536, (b, S // gs, h, 128)).astype(np.uint16),
+                    rng.integers(0, 65536, (b, S // gs, h, 128)).astype(np.uint16),
+                    rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8),
+                    rng.integers(0, 65536, (b, S, h, 1)).astype(np.uint16),
+                    rng.integers(0, 65536, (b, S, h, 1)).astype(np.uint16))
+    full = mk(256)
+    whole = L.pack_physical(*full, bits, gs)
+    for half in (0, 1):
+        part = tuple(a[:, (half * 128 // (256 // a.shape[1])):((half + 1) * 128 // (256 // a.shape[1]))] for a in full)
+        sub = L.pack_physical(*part, bits, gs)
+        for w, s_ in zip(whole, sub):
+            wb = w.reshape(-1).view(np.uint8).reshape(b * h, -1)
+            sb = s_.reshape(-1).view(np.uint8).reshape(b * h, -1)
+            n = sb.shape[1]
+            np.testing.assert_array_equal(wb[:, half * n:(half + 1) * n], sb)
+
+
+# ------------------------------------------------------------------ C ABI
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "bitdecode.h")).read()
+    declared = set(re.findall(r"\b(bitdecode_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    lib = _lib.lib()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.bitdecode_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_mirrors_match_header_field_order():
+    header = open(os.path.join(ROOT, "include", "bitdecode.h")).read()
+    for cname, cls in (("bitdecode_qpack_args", _lib.QpackArgs), ("bitdecode_fwd_args", _lib.FwdArgs)):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), header, re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        names = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            for part in decl.split(","):
+                names.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
+        assert names == [f[0] for f in cls._fields_], cname
+
+
+def _fwd_args(**kw):
+    a = _lib.FwdArgs()
+    fake = 0x1000
+    a.q = a.out = a.k_pack = a.k_params = a.v_pack = a.v_params = fake
+    a.q_stride_b, a.q_stride_h = 32 * 128, 128
+    a.out_stride_b, a.out_stride_h = 32 * 128, 128
+    a.cache_tokens = a.seqlen_k = a.max_seqlen_k = 1024
+    a.b, a.h, a.h_k, a.d = 1, 32, 8, 128
+    a.bits, a.group_size, a.dtype = 4, 128, 0
+    a.softmax_scale = 0.088
+    a.num_splits = 1
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,code,text", [
+    (dict(d=64), 2, "head_dim"),
+    (dict(bits=3), 2, "num_bits"),
+    (dict(group_size=16), 2, "group_size"),
+    (dict(dtype=5), 2, "dtype"),
+    (dict(h=30), 1, "multiple"),
+    (dict(h=8 * 9), 2, "query heads per kv head"),
+    (dict(seqlen_k=1000, max_seqlen_k=1000), 1, "multiple of 128"),
+    (dict(seqlen_k=2048, max_seqlen_k=2048), 1, "exceeds cache capacity"),
+    (dict(q=0), 1, "null"),
+    (dict(q=0x1004), 1, "aligned"),
+    (dict(q_stride_h=100), 1, "strides"),
+    (dict(num_splits=4), 3, "workspace"),
+    (dict(num_splits=-1), 1, "negative"),
+    (dict(res_len=5), 1, "null residual"),
+])
+def test_fwd_rejects_bad_arguments_without_launching(kw, code, text):
+    lib = _lib.lib()
+    rc = lib.bitdecode_fwd(ctypes.byref(_fwd_args(**kw)), None)
+    assert rc == code, lib.bitdecode_last_error()
+    assert text in lib.bitdecode_last_error().decode()
+    with pytest.raises(_lib.BitDecodeError):
+        _lib.check(rc)
+
+
+def _qpack_args(**kw):
+    a = _lib.QpackArgs()
+    fake = 0x1000
+    a.k = a.v = a.k_pack = a.k_params = a.v_pack = a.v_params = fake
+    a.k_stride_b = a.v_stride_b = 256 * 8 * 128
+    a.k_stride_t = a.v_stride_t = 8 * 128
+    a.k_stride_h = a.v_stride_h = 128
+    a.b, a.n_tokens, a.h_k, a.d = 1, 256, 8, 128
+    a.cache_tokens = 1024
+    a.bits, a.group_size, a.dtype = 4, 128, 0
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("kw,code,text", [
+    (dict(n_tokens=100), 1, "multiple of 128"),
+    (dict(cache_tokens=1000), 1, "cache_tokens"),
+    (dict(dst_offset=64), 1, "dst_offset"),
+    (dict(dst_offset=896), 1, "exceeds cache capacity"),
+    (dict(bits=8), 2, "num_bits"),
+    (dict(k=0), 1, "null"),
+    (dict(k_stride_t=1020), 1, "strides"),
+])
+def test_qpack_rejects_bad_arguments_without_launching(kw, code, text):
+    lib = _lib.lib()
+    rc = lib.bitdecode_qpack(ctypes.byref(_qpack_args(**kw)), None)
+    assert rc == code, lib.bitdecode_last_error()
+    assert text in lib.bitdecode_last_error().decode()
+
+
+def test_qpack_of_zero_tokens_is_a_no_op():
+    assert _lib.lib().bitdecode_qpack(ctypes.byref(_qpack_args(n_tokens=0)), None) == 0
+
+
+def test_split_choice_and_workspace_size():
+    lib = _lib.lib()
+    # 32K GQA config on 256 CUs: 8 kv heads x 32 splits = one workgroup per CU, one chunk per wave
+    assert lib.bitdecode_num_splits(1, 8, 32768, 128, 256) == 32
+    # enough (batch x kv-head) workgroups already: no split
+    assert lib.bitdecode_num_splits(64, 8, 4096, 128, 256) == 1
+    # never more splits than there is work for
+    assert lib.bitdecode_num_splits(1, 1, 256, 0, 256) == 1
+    assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256) == 3
+    assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
+    assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 256 + 32 * 32 * 129 * 4
+
+
+def test_python_entry_points_validate_before_touching_the_gpu():
+    import torch
+    from bitladder_amd import fwd_kvcache_int, kvcache_pack_int
+    t = torch.zeros(1, 128, 2, 128, dtype=torch.float16)
+    kp = torch.zeros(1, 32, 2, 128, dtype=torch.uint16)
+    with pytest.raises(NotImplementedError):
+        kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-tensor", 128, 4)
+    with pytest.raises(ValueError):
+        kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-channel", 48, 4)
+    with pytest.raises(ValueError):
+        fwd_kvcache_int(t[:, :1], kp, kp, kp, kp, None, 1.0, "k-channel", 128, 3)
+    with pytest.raises(NotImplementedError):
+        fwd_kvcache_int(t[:, :1], kp, kp, kp, kp, torch.zeros(1, 1, dtype=torch.int32))
+    with pytest.raises(RuntimeError):      # CPU tensors: the reference's CHECK_DEVICE
+        kvcache_pack_int(t, kp, kp, t, kp, kp)
+
+
+def test_drop_in_package_name_and_signatures():
+    import inspect
+    import bit_decode
+    sig = inspect.signature(bit_decode.kvcache_pack_int)
+    assert list(sig.parameters)[:12] == ["k_cache", "k_pack", "k_params", "v_cache", "v_pack", "v_params",
+                                         "opt_block_table", "cu_seqlens_k", "seqlen_k", "quant_mode", "group_size",
+                                         "num_bits"]
+    assert sig.parameters["group_size"].default == 128 and sig.parameters["num_bits"].default == 4
+    sig = inspect.signature(bit_decode.fwd_kvcache_int)
+    assert list(sig.parameters)[:10] == ["q", "k_pack", "k_params", "v_pack", "v_params", "opt_block_table",
+                                         "softmax_scale", "quant_mode", "group_size", "num_bits"]
+    assert sig.parameters["softmax_scale"].default == 1.0       # bit_decode_interface.py:47
+    assert bit_decode.__version__ == "1.0.0.post1"              # bit_decode/__init__.py:1
