@@ -22,6 +22,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the split-KV kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/fwd_splitkv_llama3-8b-gqa-32k-4bit-g128.md): the counters read 18090.8 and 560.25 per
+# dispatch; a 256 MiB device copy in the same runs reads 131089 and 262144, i.e. the fetch counter
+# is in units of 2 KiB and the write counter in KiB.
+MEASURED_TRAFFIC_BYTES = {
+    "llama3-8b-gqa-32k-4bit-g128": int(18090.8 * 2048 + 560.25 * 1024),
+}
+
 WORKLOADS = {
     # name: (b, h, h_k, S, R, bits, gs, dtype)
     "llama3-8b-gqa-32k-4bit-g128": (1, 32, 8, 32768, 128, 4, 128, torch.float16),
@@ -126,6 +134,9 @@ def main():
     ap.add_argument("--no-rotate", action="store_true", help="reuse one KV cache (stays in the 256 MB Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fp16", action="store_true", help="skip the fp16-KV baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch three plain 256 MiB device copies (a kernel of known traffic, used to scale "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this decode path has no cross-GPU step (it shards by kv-head / batch "
@@ -167,6 +178,14 @@ def main():
     def step(i):
         plans[i % nbuf].run()
 
+    if args.calib_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize(dev)
+        del src, dst
+
     wall, evs, graphed = time_steps(step, args.steps, args.warmup, not args.no_graph)
     us_step = wall / args.steps * 1e6
     us_step_ev = evs / args.steps * 1e6
@@ -192,7 +211,8 @@ def main():
                    "num_splits": plans[0].num_splits, "kv_buffers_rotated": nbuf,
                    "launch": "hip-graph" if graphed else "eager"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.num_splits == 0 else None,
                      "kernel": "fwd_splitkv_kernel", "algorithmic_bytes": total_bytes,
                      "packed_stream_bytes": packed_bytes, "us_per_step_events": round(us_step_ev, 3)},
     }
