@@ -78,7 +78,7 @@ def lib():
         L.bitdecode_abi_version.restype = ctypes.c_int
         L.bitdecode_last_error.restype = ctypes.c_char_p
         L.bitdecode_num_splits.restype = ctypes.c_int
-        L.bitdecode_num_splits.argtypes = [_i32] * 5
+        L.bitdecode_num_splits.argtypes = [_i32] * 7
         L.bitdecode_fwd_workspace_bytes.restype = ctypes.c_size_t
         L.bitdecode_fwd_workspace_bytes.argtypes = [_i32] * 3
         L.bitdecode_qpack.restype = ctypes.c_int

@@ -44,17 +44,19 @@ int query_cus() {
     return n;
 }
 
-// A wave streams whole 128-token packed chunks (plus a share of the 16-token fp16 tiles) and a
-// workgroup has 8 waves.  Pick the number of splits so that the grid is about one workgroup per CU
-// while every wave still gets at least one chunk (or four fp16 tiles when nothing is packed).
-int choose_splits(int b, int hk, int max_seqlen_k, int max_res_len, int num_cus) {
-    const int chunks = max_seqlen_k / bitdecode::kChunk;
+// A wave streams whole packed units (64 tokens at 4 bits, 128 at 2 bits) plus a share of the 16-token
+// fp16 tiles, and a workgroup has 16 or 12 waves.  Pick the number of splits so that the grid is about
+// one workgroup per CU while every wave still gets at least one unit (or four fp16 tiles when nothing
+// is packed).
+int choose_splits(int b, int hk, int max_seqlen_k, int max_res_len, int num_cus, int bits, int gs) {
+    const int nw = bitdecode::decode_waves(bits, gs);
+    const int packed_units = max_seqlen_k / bitdecode::unit_tokens(bits);
     const int tiles = (max_res_len + 15) / 16;
-    const int units = chunks > 0 ? chunks : (tiles + 3) / 4;
+    const int units = packed_units > 0 ? packed_units : (tiles + 3) / 4;
     if (units <= 0) return 1;
     const int heads = std::max(1, b * hk);
     const int by_occupancy = std::max(1, (num_cus + heads - 1) / heads);
-    const int by_work = std::max(1, (units + 7) / 8);
+    const int by_work = std::max(1, (units + nw - 1) / nw);
     int n = std::min(std::min(by_occupancy, by_work), 256);
     // drop splits that would be empty: ceil(units / n) units per split
     const int ups = (units + n - 1) / n;
@@ -70,9 +72,11 @@ int bitdecode_abi_version(void) { return BITDECODE_ABI_VERSION; }
 
 const char* bitdecode_last_error(void) { return g_err; }
 
-int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len, int32_t num_cus) {
+int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len, int32_t num_cus,
+                         int32_t bits, int32_t group_size) {
     if (num_cus <= 0) num_cus = query_cus();
-    return choose_splits(b, h_k, max_seqlen_k, max_res_len, num_cus);
+    if (check_quant(bits, group_size, BITDECODE_FP16, bitdecode::kHeadDim)) return -1;
+    return choose_splits(b, h_k, max_seqlen_k, max_res_len, num_cus, bits, group_size);
 }
 
 // [tickets: b*h ints rounded up to 256 B][o_part][lse_part]
@@ -161,7 +165,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
 
     int nsplit = a->num_splits;
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
-    if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus());
+    if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
     if (nsplit > 1) {
         const size_t need = bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
         if (!a->workspace || a->workspace_bytes < need)
@@ -194,6 +198,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     P.scale = a->softmax_scale;
     P.scale_log2 = fabsf(a->softmax_scale) * 1.4426950408889634f;   // decode_api.cpp:128-142
     P.neg_scale = a->softmax_scale < 0.0f;
+    P.xcd_remap = (a->b * a->h_k) % 8 == 0 && nsplit > 1;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
     if (nsplit > 1) {
         P.tickets = static_cast<int*>(a->workspace);

@@ -3,9 +3,13 @@
 // Replaces compute_attn_1rowblock_splitkv and combine_attn_seqk_parallel of the reference
 // (csrc/bit_decode/src/flash_fwd_kernel.h:66-728, 1144-1327) with a wave64/MFMA design:
 //
-//  * A workgroup owns one (split, kv-head, batch); each of its waves streams whole work units of
-//    that split: a packed 128-token chunk (~17 KB at 4 bits) or a 32-token fp16 block (16 KB).
-//    All chunk data is fetched with 16-byte lane loads that form contiguous 1 KB wave rows.
+//  * A workgroup owns one (split, kv-head, batch).  Each wave streams whole work units of that
+//    split: 64 packed tokens at 4 bits / 128 at 2 bits (about 9 KB with their parameters), or
+//    16-token tiles of the fp16 window.  A unit is fetched with nine direct-to-LDS loads
+//    (global_load_lds_dwordx4: 64 lanes x 16 B = one contiguous 1 KB row each, no staging
+//    registers) into the wave's private LDS region and read back 16 bytes per lane just before
+//    it is unpacked.  With no load-staging registers the kernel fits 3-4 waves per SIMD, which is
+//    what hides the load latency: a wave that waits for its unit leaves the VALU to the others.
 //  * Both products are computed transposed on v_mfma_f32_16x16x32_f16:
 //        S^T = K * Q^T   (A = K codes, row = token; B = Q, column = query head of the GQA group)
 //        O^T = V^T * P^T (A = V codes, row = channel; B = P^T)
@@ -59,8 +63,7 @@ __device__ unsigned long long* g_prof = nullptr;
     do {                                                                                              \
         unsigned long long* pb = g_prof;                                                              \
         if (pb && (threadIdx.x & 63) == 0) {                                                          \
-            pb += ((((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * kNW +   \
-                   (threadIdx.x >> 6)) * 8;                                                           \
+            pb += ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 8;                                  \
             for (int i_ = 0; i_ < 8; ++i_) pb[i_] = prof_ts[i_];                                      \
         }                                                                                             \
     } while (0)
@@ -70,7 +73,6 @@ __device__ unsigned long long* g_prof = nullptr;
 #define PROF_FLUSH() do { } while (0)
 #endif
 
-constexpr int kNW = 8;            // waves per workgroup
 constexpr float kPShift = 2.0f;   // probabilities are kept as 2^kPShift * exp2(s - max): a V scale
                                   // is at most 65504*2/3, so p*scale cannot overflow fp16
 constexpr int kLdsRowHalves = 136;
@@ -225,165 +227,249 @@ __device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveSta
 }
 
 // ---------------------------------------------------------------------------------------------
-// packed 128-token chunks
+// packed units, streamed through LDS
 // ---------------------------------------------------------------------------------------------
-// Registers holding one chunk's global loads.  K side and V side are separate so that the next
-// chunk's K loads can be issued as soon as this chunk's K registers are consumed (and likewise
-// for V): with one chunk per wave every load of the kernel is in flight from the first cycle.
 template <int BITS, int GS>
-struct KSide {
-    static constexpr int NG = kChunk / GS;
-    static constexpr int NW4 = BITS == 4 ? 8 : 4;     // 16-byte lane loads of codes per chunk
-    static constexpr int PF = NG <= 2 ? NG : 1;       // parameter groups fetched with the chunk
-    u4 code[NW4];
-    u4 ps[PF][4], pz[PF][4];
-};
-template <int BITS, int GS>
-struct VSide {
-    static constexpr int NCG = kHeadDim / GS;
-    static constexpr int NW4 = BITS == 4 ? 8 : 4;
-    static constexpr int PF = NCG == 1 ? 4 : 0;       // sub-blocks whose params are fetched with the chunk
-    u4 code[NW4];
-    u4 ps[PF ? PF : 1], pz[PF ? PF : 1];
+struct UnitCfg {
+    static constexpr int UT = unit_tokens(BITS);             // tokens per unit (4 KB of K codes, 4 KB of V codes)
+    static constexpr int UPC = kChunk / UT;                  // units per 128-token chunk
+    static constexpr int NTILE = UT / 16;                    // 16-token tiles per unit
+    static constexpr int TPS = NTILE / 2;                    // tiles per step (two steps per unit)
+    static constexpr int NKS = TPS / 2;                      // 32-token k-steps (V sub-blocks) per step
+    static constexpr int TPG = GS / 16;                      // tiles per K group
+    static constexpr int NGU = UT > GS ? UT / GS : 1;        // K groups a unit touches
+    static constexpr int NCG = kHeadDim / GS;                // V channel groups
+    static constexpr int KPB = NGU * kKParamGroupBytes;      // K parameter bytes per unit
+    static constexpr int VPB = UT * NCG * 4;                 // V parameter bytes per unit
+    static constexpr int PROWS = (KPB + VPB + 1023) / 1024;  // 1 KB rows holding [K params | V params]
+    static constexpr int REGION = 8192 + PROWS * 1024;       // LDS bytes per wave: K codes, V codes, params
+    static constexpr int NW = decode_waves(BITS, GS);        // waves per workgroup
+    static_assert(REGION == unit_region_bytes(BITS, GS), "layout.h and the kernel disagree on the LDS region");
 };
 
-template <int BITS, int GS>
-__device__ __forceinline__ void load_kside(KSide<BITS, GS>& K, const FwdParams& P, int64_t bh, int ci, int lane) {
-    constexpr int NG = kChunk / GS;
-    const int kg = lane >> 4;
-    const uint8_t* kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
-    const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
-    const uint32_t poff = kg * 16, coff = lane * 16;     // per-lane byte offsets from uniform bases
-#pragma unroll
-    for (int g = 0; g < KSide<BITS, GS>::PF; ++g) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            K.ps[g][j] = ld_u4(kp + (g * kKParamGroupBytes + 64 * j) + poff);
-            K.pz[g][j] = ld_u4(kp + (g * kKParamGroupBytes + 256 + 64 * j) + poff);
-        }
-    }
-#pragma unroll
-    for (int x = 0; x < KSide<BITS, GS>::NW4; ++x) K.code[x] = ld_u4(kc + x * 1024 + coff);
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_base + 16*l.
+// M0 carries the LDS byte address of the row.
+__device__ __forceinline__ void dma_row(const void* gaddr_of_lane, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gaddr_of_lane), "s"(lds_base)
+                 : "memory", "m0");
 }
 
-template <int BITS, int GS>
-__device__ __forceinline__ void load_vside(VSide<BITS, GS>& V, const FwdParams& P, int64_t bh, int ci, int lane) {
-    const int kg = lane >> 4;
-    const uint8_t* vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS);
-    const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
-    const uint32_t poff = kg * 16, coff = lane * 16;
-#pragma unroll
-    for (int sb = 0; sb < VSide<BITS, GS>::PF; ++sb) {
-        V.ps[sb] = ld_u4(vp + sb * 128 + poff);
-        V.pz[sb] = ld_u4(vp + (sb * 128 + 64) + poff);
-    }
-#pragma unroll
-    for (int x = 0; x < VSide<BITS, GS>::NW4; ++x) V.code[x] = ld_u4(vc + x * 1024 + coff);
+// s_waitcnt vmcnt(n): at most n of this wave's loads still in flight.  The compiler does not
+// track the asm loads above, so the waits are explicit; the memory clobber keeps LDS reads below.
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// One packed chunk in steps of 32 tokens (4-bit) or 64 tokens (2-bit): S^T tiles of the step,
-// online-softmax update, O^T += V^T P^T for the same tokens.  Scores stay in q.k units; the
-// softmax scale is applied inside the exponent.
+// A 16-byte global load the compiler does not track (so that its automatic waits do not count
+// the direct-to-LDS loads above as its own).  The loaded registers must not be touched before the
+// matching wait_then_take, which waits and only then copies them into registers the compiler may
+// use freely: the copy happens inside the same asm block as the wait, so nothing can be scheduled
+// between them.
+__device__ __forceinline__ u4 load_untracked(const void* gaddr) {
+    u4 r;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(gaddr) : "memory");
+    return r;
+}
+template <int N>
+__device__ __forceinline__ void wait_then_take(u4& dst_a, u4& dst_b, const u4& a, const u4& b) {
+    typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+    u2 a0, a1, b0, b1;
+    asm volatile(
+        "s_waitcnt vmcnt(%8)\n\t"
+        "v_mov_b64 %0, %4\n\t"
+        "v_mov_b64 %1, %5\n\t"
+        "v_mov_b64 %2, %6\n\t"
+        "v_mov_b64 %3, %7"
+        : "=&v"(a0), "=&v"(a1), "=&v"(b0), "=&v"(b1)
+        : "v"(u2{a[0], a[1]}), "v"(u2{a[2], a[3]}), "v"(u2{b[0], b[1]}), "v"(u2{b[2], b[3]}), "n"(N)
+        : "memory");
+    dst_a = u4{a0[0], a0[1], a1[0], a1[1]};
+    dst_b = u4{b0[0], b0[1], b1[0], b1[1]};
+}
+
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (const __attribute__((address_space(3))) void*)p));
+}
+
+// The loads of unit u, in the order they are consumed.  First half: params, K rows 0-1, V rows 0-1
+// (step 0); second half: K rows 2-3, V rows 2-3 (step 1).  The second half is issued while step 0
+// is being computed: a wave stalls while the memory pipeline will not take its next load, so it
+// only queues what it needs next and keeps the VALU busy in between.
+template <int BITS, int GS>
+struct UnitAddr {
+    const uint8_t* kc;
+    const uint8_t* vc;
+    const uint8_t* kp;
+    const uint8_t* vp;
+};
+template <int BITS, int GS>
+__device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int64_t bh, int u, int lane) {
+    using C = UnitCfg<BITS, GS>;
+    const int ci = u / C::UPC, uic = u % C::UPC;
+    UnitAddr<BITS, GS> A;
+    A.kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096 + lane * 16;
+    A.vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096 + lane * 16;
+    A.kp = P.k_params + bh * P.kparams_bh +
+           (static_cast<int64_t>(ci) * (kChunk / GS) + (uic * C::UT) / GS) * kKParamGroupBytes;
+    A.vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS) + uic * C::VPB;
+    return A;
+}
+template <int BITS, int GS>
+__device__ __forceinline__ void issue_first_half(const UnitAddr<BITS, GS>& A, int lane, uint32_t region) {
+    using C = UnitCfg<BITS, GS>;
+#pragma unroll
+    for (int r = 0; r < C::PROWS; ++r) {
+        const int o = r * 1024 + lane * 16;                   // byte offset inside [K params | V params]
+        const uint8_t* src =
+            o < C::KPB ? A.kp + o : (o < C::KPB + C::VPB ? A.vp + (o - C::KPB) : A.kp + (o & (C::KPB - 1)));
+        dma_row(src, region + 8192 + r * 1024);
+    }
+    dma_row(A.kc, region);
+    dma_row(A.kc + 1024, region + 1024);
+    dma_row(A.vc, region + 4096);
+    dma_row(A.vc + 1024, region + 4096 + 1024);
+}
+template <int BITS, int GS>
+__device__ __forceinline__ void issue_second_half(const UnitAddr<BITS, GS>& A, uint32_t region) {
+    dma_row(A.kc + 2048, region + 2048);
+    dma_row(A.kc + 3072, region + 3072);
+    dma_row(A.vc + 2048, region + 4096 + 2048);
+    dma_row(A.vc + 3072, region + 4096 + 3072);
+}
+
+// Per-group state of the K side: Q with the group's scale folded in (exact hi/lo split) and the
+// score bias  sum_c q_c*zero_c - sum_c (q_c*scale_c)*offset_c  built on the MFMA pipe.
+struct KGroup {
+    h8 qp[4];
+    f4 kb;
+};
+
+// The workgroup's LDS copy of q: rows 0-7 = the eight head slots of the GQA group ([128] fp16
+// values each; slots past the group repeat head 0 and are never written out), row 8 = zeros.
+// A lane reads q three ways without any select: plain (its head), hi-only (zero row in the lo
+// columns) and lo-only (zero row in the hi columns).
+struct QRows {
+    const uint8_t* q;    // row of this lane's head
+    const uint8_t* qz;   // same row in the hi columns, zero row in the lo columns
+    const uint8_t* qm;   // zero row in the hi columns, same row in the lo columns
+};
+__device__ __forceinline__ QRows q_rows(const uint8_t* sq, int head, int kg, bool lo_part) {
+    const uint8_t* row = sq + head * 256 + kg * 16;
+    const uint8_t* zero = sq + 8 * 256 + kg * 16;
+    return QRows{row, lo_part ? zero : row, lo_part ? row : zero};
+}
+__device__ __forceinline__ h8 q_load(const uint8_t* row, int j) {
+    return __builtin_bit_cast(h8, *reinterpret_cast<const u4*>(row + 64 * j));
+}
+
+// a*b as an exact fp16 pair: hi columns get hi = round(a*b), lo columns get fma(a, b, -hi).
+// a_lo_only is a in the lo columns and 0 in the hi columns, so no lane select is needed.
+__device__ __forceinline__ h8 split_mul_masked(h8 a, h8 a_lo_only, h8 b) {
+    const h8 hi_in_lo_cols = a_lo_only * b;
+    return __builtin_elementwise_fma(a, b, -hi_in_lo_cols);
+}
+
+template <int BITS, bool BF16>
+__device__ __forceinline__ void start_group(KGroup& G, const uint8_t* kpar, const QRows& Q, int kg) {
+    const h8 noff = -code_offsets<BITS>();
+    G.kb = f4{0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const h8 sc = cvt_h8<false>(*reinterpret_cast<const u4*>(kpar + (32 * j + 8 * kg) * 2));
+        const h8 zr = cvt_h8<false>(*reinterpret_cast<const u4*>(kpar + 256 + (32 * j + 8 * kg) * 2));
+        G.qp[j] = split_mul_masked(q_load(Q.q, j), q_load(Q.qm, j), sc);
+        G.kb = mfma32(zr, q_load(Q.qz, j), G.kb);
+        G.kb = mfma32(noff, G.qp[j], G.kb);
+    }
+}
+
+// One packed unit from the wave's LDS region, in two steps: S^T tiles of the step, online
+// softmax update, O^T += V^T P^T for the same tokens.  Scores stay in q.k units; the softmax
+// scale is applied inside the exponent.  `pending` = loads issued after this unit's (0 here).
 template <int BITS, int GS, bool BF16>
-__device__ __forceinline__ void packed_chunk(const KSide<BITS, GS>& K, const VSide<BITS, GS>& V, const FwdParams& P,
-                                             int64_t bh, int ci, int lane, const h8 (&qB)[4], bool lo_part,
+__device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, const UnitAddr<BITS, GS>& A,
+                                             const QRows& Q, const FwdParams& P, int lane, bool lo_part,
                                              const Magic& mg, WaveState<kHeadDim / GS>& st) {
-    constexpr int NG = kChunk / GS;
-    constexpr int NCG = kHeadDim / GS;
-    constexpr int TPG = GS / 16;                 // 16-token tiles per K group
-    constexpr int CTPG = GS / 16;                // 16-channel tiles per V channel group
-    constexpr int TPS = BITS == 4 ? 2 : 4;       // tiles per step
-    constexpr int NSTEP = 8 / TPS;
-    constexpr int KPF = KSide<BITS, GS>::PF;
-    constexpr int VPF = VSide<BITS, GS>::PF;
+    using C = UnitCfg<BITS, GS>;
+    constexpr int NCG = C::NCG, TPS = C::TPS, NKS = C::NKS, TPG = C::TPG, CTPG = GS / 16;
     const int kg = lane >> 4;
     const h8 noff = -code_offsets<BITS>();
     const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
-    const h8 zero8 = h8{0, 0, 0, 0, 0, 0, 0, 0};
-    const uint8_t* kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * NG * kKParamGroupBytes;
-    const uint8_t* vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS);
+    const bool neg = P.neg_scale != 0;
+    const uint32_t hi_cols = lo_part ? 0u : 0xffffffffu;
+    const u4* kcode = reinterpret_cast<const u4*>(reg) + lane;             // row r: kcode[64 * r]
+    const u4* vcode = reinterpret_cast<const u4*>(reg + 4096) + lane;
+    const uint8_t* kpar = reg + 8192;
+    const uint8_t* vpar = reg + 8192 + C::KPB + kg * 16;
 
-    h8 qp[4];
-    f4 kb = {0, 0, 0, 0};
+    KGroup G;
 #pragma unroll
-    for (int step = 0; step < NSTEP; ++step) {
+    for (int step = 0; step < 2; ++step) {
+        // loads still allowed in flight when the K rows of this step are needed: its two V rows
+        wait_vm<2>();
         float t[4 * TPS];
 #pragma unroll
         for (int tt = 0; tt < TPS; ++tt) {
             const int tile = step * TPS + tt;
-            if (tile % TPG == 0) {
-                // new K group: fold its scale into Q (exact hi/lo split) and build the score bias
-                // sum_c q_c*zero_c - sum_c (q_c*scale_c)*offset_c on the MFMA pipe
-                const int grp = tile / TPG;
-                kb = f4{0, 0, 0, 0};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    u4 rs, rz;
-                    if (grp < KPF) {
-                        rs = K.ps[grp < KPF ? grp : 0][j];
-                        rz = K.pz[grp < KPF ? grp : 0][j];
-                    } else {
-                        rs = ld_u4(kp + (grp * kKParamGroupBytes + 64 * j) + kg * 16);
-                        rz = ld_u4(kp + (grp * kKParamGroupBytes + 256 + 64 * j) + kg * 16);
-                    }
-                    qp[j] = split_mul(qB[j], cvt_h8<BF16>(rs), lo_part);
-                    kb = mfma32(cvt_h8<BF16>(rz), lo_part ? zero8 : qB[j], kb);
-                    kb = mfma32(noff, qp[j], kb);
-                }
+            if (tile == 0 || tile % TPG == 0) {
+                start_group<BITS, BF16>(G, kpar + ((tile * 16) / GS) * kKParamGroupBytes * (C::NGU > 1 ? 1 : 0), Q, kg);
             }
-            f4 acc = kb;
+            f4 acc = G.kb;
             if constexpr (BITS == 4) {
-                const u4 w = K.code[tile];
+                const u4 w = kcode[64 * tile];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc = mfma32(dq4(w[j], mg), qp[j], acc);
+                for (int j = 0; j < 4; ++j) acc = mfma32(dq4(w[j], mg), G.qp[j], acc);
             } else {
-                const u4 w = K.code[tile / 2];
+                const u4 w = kcode[64 * (tile / 2)];
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
                     h8 a0, a1;
                     dq2(w[2 * (tile % 2) + jj], a0, a1, mg);
-                    acc = mfma32(a0, qp[2 * jj], acc);
-                    acc = mfma32(a1, qp[2 * jj + 1], acc);
+                    acc = mfma32(a0, G.qp[2 * jj], acc);
+                    acc = mfma32(a1, G.qp[2 * jj + 1], acc);
                 }
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) t[4 * tt + r] = acc[r] + partner(acc[r]);   // hi + lo
         }
+        if (step == 0) issue_second_half<BITS, GS>(A, region_lds);
+        if (neg) {      // softmax_scale < 0: scale_log2 holds |scale|, the sign goes into the scores
+#pragma unroll
+            for (int i = 0; i < 4 * TPS; ++i) t[i] = -t[i];
+        }
 
         softmax_step<4 * TPS, NCG>(t, P.scale_log2, st);
 
-        // ---- O^T += V^T P^T for the tokens of this step
-        constexpr int NKS = TPS / 2;                  // 32-token k-steps in this step
-        h8 p16[NKS], pz[NKS];
+        h8 p16[NKS], pz[NKS], pm[NKS];
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
+            u4 pw;
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
                 // element i = 4*T + r  <->  tile 2*ks + T of the step, accumulator register r
-                const h2 pr = pk_rtz(t[8 * ks + 2 * x], t[8 * ks + 2 * x + 1]);
-                p16[ks][2 * x] = pr[0];
-                p16[ks][2 * x + 1] = pr[1];
+                pw[x] = __builtin_bit_cast(uint32_t, pk_rtz(t[8 * ks + 2 * x], t[8 * ks + 2 * x + 1]));
             }
-            pz[ks] = lo_part ? zero8 : p16[ks];       // p itself only in the hi columns
+            p16[ks] = __builtin_bit_cast(h8, pw);
+            pz[ks] = __builtin_bit_cast(h8, pw & hi_cols);       // p itself only in the hi columns
+            pm[ks] = __builtin_bit_cast(h8, pw & ~hi_cols);      // and only in the lo columns
             st.l = mfma32(ones, pz[ks], st.l);
         }
-        const u4 w0 = V.code[2 * step], w1 = V.code[2 * step + 1];
+        if (step == 0) wait_vm<4>(); else wait_vm<0>();
+        const u4 w0 = vcode[64 * (2 * step)], w1 = vcode[64 * (2 * step + 1)];
 #pragma unroll
         for (int cg = 0; cg < NCG; ++cg) {
             h8 pp[NKS];
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
-                const int sb = step * NKS + ks;
-                u4 rs, rz;
-                if (VPF) {
-                    rs = V.ps[VPF ? sb : 0];
-                    rz = V.pz[VPF ? sb : 0];
-                } else {
-                    rs = ld_u4(vp + (sb * NCG + cg) * 128 + kg * 16);
-                    rz = ld_u4(vp + ((sb * NCG + cg) * 128 + 64) + kg * 16);
-                }
-                pp[ks] = split_mul(p16[ks], cvt_h8<BF16>(rs), lo_part);
-                st.ob[cg] = mfma32(cvt_h8<BF16>(rz), pz[ks], st.ob[cg]);
+                const int sb = step * NKS + ks;               // 32-token sub-block inside the unit
+                const u4 rs = *reinterpret_cast<const u4*>(vpar + (sb * NCG + cg) * 128);
+                const u4 rz = *reinterpret_cast<const u4*>(vpar + (sb * NCG + cg) * 128 + 64);
+                pp[ks] = split_mul_masked(p16[ks], pm[ks], cvt_h8<false>(rs));
+                st.ob[cg] = mfma32(cvt_h8<false>(rz), pz[ks], st.ob[cg]);
                 st.ob[cg] = mfma32(noff, pp[ks], st.ob[cg]);
             }
 #pragma unroll
@@ -432,9 +518,8 @@ __device__ __forceinline__ void load_fp16_tile(Fp16Tile& T, const FwdParams& P, 
 
 template <bool BF16, int NCG>
 __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P, int n0, int R, int lane,
-                                          const h8 (&qB)[4], bool lo_part, WaveState<NCG>& st, uint16_t* lds) {
+                                          const QRows& Q, bool lo_part, WaveState<NCG>& st, uint16_t* lds) {
     const int col = lane & 15, kg = lane >> 4;
-    const h8 zero8 = h8{0, 0, 0, 0, 0, 0, 0, 0};
 
     // V tile (16 tokens x 128 channels) goes through this wave's LDS slab to be read back
     // token-contiguous per channel (the MFMA A operand wants 4 tokens of one channel per lane).
@@ -451,12 +536,13 @@ __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P,
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             // fp16 operands are exact: only the hi columns carry q
-            acc = mfma32(cvt_h8<BF16>(T.k[j]), lo_part ? zero8 : qB[j], acc);
+            acc = mfma32(cvt_h8<BF16>(T.k[j]), q_load(Q.qz, j), acc);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int tk = n0 + 4 * kg + r;
-            const float tot = acc[r] + partner(acc[r]);   // outside the select: every lane executes the DPP
+            float tot = acc[r] + partner(acc[r]);   // outside the select: every lane executes the DPP
+            if (P.neg_scale) tot = -tot;
             s[r] = tk < R ? tot : -INFINITY;
         }
     }
@@ -506,28 +592,55 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// split-KV kernel: grid (num_splits, h_k, b), kNW waves.
-// Split s of a (batch, kv-head) owns packed chunks [s*cps, (s+1)*cps) dealt round-robin to its
+// split-KV kernel: 1-D grid of num_splits * h_k * b workgroups of UnitCfg::NW waves.
+// Split s of a (batch, kv-head) owns packed units [s*ups, (s+1)*ups) dealt round-robin to its
 // waves; the 16-token tiles of the fp16 window are dealt round-robin over ALL waves of the head.
 // With more than one split each workgroup writes a normalised partial and takes a ticket; the
 // workgroup that draws the last ticket of its (batch, kv-head) merges all partials
 // (flash_fwd_kernel.h:1217-1298 formula) and resets the ticket.
+//
+// Dynamic LDS: [NW wave regions of UnitCfg::REGION bytes][q: 8 head rows + a zero row, 256 B each][sM, sL: NW x 8 floats]
+// A wave's region is reused as its V-transpose slab for fp16 tiles and as its slot of the
+// cross-wave merge buffer (g x 128 floats <= 4 KB).
 // ---------------------------------------------------------------------------------------------
+template <int BITS, int GS>
+constexpr int fwd_lds_bytes() {
+    using C = UnitCfg<BITS, GS>;
+    return C::NW * C::REGION + (kMaxGroupHeads + 1) * 256 + 2 * C::NW * kMaxGroupHeads * 4 + 16;
+}
+
 template <int BITS, int GS, bool BF16>
-__global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
-    constexpr int NCG = kHeadDim / GS;
-    constexpr int kSlabHalves = 16 * kLdsRowHalves;
-    constexpr int kMergeFloats = kNW * kMaxGroupHeads * kHeadDim;
-    constexpr int kLdsBytes = (kMergeFloats * 4 > kNW * kSlabHalves * 2) ? kMergeFloats * 4 : kNW * kSlabHalves * 2;
-    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kLdsBytes];
-    __shared__ float sM[kNW][kMaxGroupHeads], sL[kNW][kMaxGroupHeads];
-    __shared__ int s_last;
+__global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
+    using C = UnitCfg<BITS, GS>;
+    constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t* const sq = lds + NW * REGION;                                   // [8 + zero row][128] 16-bit q
+    float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * 256);   // [NW][8]
+    float* const sL = sM + NW * kMaxGroupHeads;
+    int* const s_last = reinterpret_cast<int*>(sL + NW * kMaxGroupHeads);
 
     PROF_DECL;
     PROF(0);
-    const int split = blockIdx.x, hk = blockIdx.y, bi = blockIdx.z;
+    // Workgroups are handed to the 8 XCDs round-robin by linear id.  When the number of
+    // (batch, kv-head) pairs is a multiple of 8, ids are remapped so that all splits of one pair run
+    // on one XCD.
+    int split, hk, bi;
+    {
+        const int lin = blockIdx.x;
+        int bhid;
+        if (P.xcd_remap) {
+            const int xcd = lin & 7, r = lin >> 3;
+            bhid = (r / P.nsplit) * 8 + xcd;
+            split = r % P.nsplit;
+        } else {
+            bhid = lin / P.nsplit;
+            split = lin % P.nsplit;
+        }
+        bi = bhid / P.hk;
+        hk = bhid % P.hk;
+    }
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: chunk addresses stay in SGPRs
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: unit addresses stay in SGPRs
     const int col = lane & 15, kg = lane >> 4;
     const int head = col & 7;          // query head inside the GQA group
     const bool lo_part = col >= 8;     // columns 8-15 carry the lo halves of the split products
@@ -536,28 +649,41 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
 
     const int S = P.seqlens ? P.seqlens[bi] : P.seqlen;
     const int R = P.reslens ? P.reslens[bi] : P.reslen;
-    const int nP = S / kChunk;
-    const int cps = (nP + P.nsplit - 1) / P.nsplit;
-    const int c0 = min(nP, split * cps);
-    const int c1 = min(nP, c0 + cps);
+    const int nU = (S / kChunk) * C::UPC;
+    const int ups = (nU + P.nsplit - 1) / P.nsplit;
+    const int u0 = min(nU, split * ups);
+    const int u1 = min(nU, u0 + ups);
     const int nT = (R + 15) / 16;
 
-    // Q is fetched unconditionally (padding columns re-read head 0 and are zeroed after the
-    // chunk loads have been issued) so that no wait sits in front of the big loads.
-    u4 qraw[4];
+    uint8_t* const region = lds + wave * REGION;
+    const uint32_t region_lds = lds_addr(region);
+
+    // ---- every wave fetches q itself (two 16-byte loads per lane cover the eight head slots),
+    // sends out the loads of its first unit, and then writes q, converted to fp16, to the
+    // workgroup's LDS copy.  All waves write identical bytes, so no barrier is needed: q is the
+    // oldest entry of each wave's own load queue.
+    int u = u0 + wave;
+    u4 qa_raw, qb_raw, qa, qb;
     {
-        const uint16_t* qp = P.q + bi * P.q_sb + (hk * g + (head < g ? head : 0)) * P.q_sh + 8 * kg;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qraw[j] = ld_u4(qp + 32 * j);
+        const int hq = lane >> 4;                         // head within a row of four
+        const uint16_t* q0 = P.q + bi * P.q_sb + (hk * g) * P.q_sh + (lane & 15) * 8;
+        qa_raw = load_untracked(q0 + (hq < g ? hq : 0) * P.q_sh);
+        qb_raw = load_untracked(q0 + (hq + 4 < g ? hq + 4 : 0) * P.q_sh);
     }
-    auto q_operand = [&](h8 (&qB)[4]) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (head >= g) qraw[j] = u4{0, 0, 0, 0};
-            qB[j] = cvt_h8<BF16>(qraw[j]);
-            if (P.neg_scale) qB[j] = -qB[j];     // scale_log2 holds |scale|: running max needs scale >= 0
-        }
-    };
+    UnitAddr<BITS, GS> A;
+    if (u < u1) {
+        A = unit_addr<BITS, GS>(P, bh, u, lane);
+        issue_first_half<BITS, GS>(A, lane, region_lds);
+        wait_then_take<C::PROWS + 4>(qa, qb, qa_raw, qb_raw);
+    } else {
+        wait_then_take<0>(qa, qb, qa_raw, qb_raw);
+    }
+    *reinterpret_cast<h8*>(sq + lane * 16) = cvt_h8<BF16>(qa);
+    *reinterpret_cast<h8*>(sq + 1024 + lane * 16) = cvt_h8<BF16>(qb);
+    if (lane < 16) *reinterpret_cast<u4*>(sq + 8 * 256 + lane * 16) = u4{0, 0, 0, 0};
+    // (head slots past the group hold head 0 again: finite values whose results are never stored)
+    const QRows Q = q_rows(sq, head, kg, lo_part);
+    PROF(1);
 
     WaveState<NCG> st;
     st.m = -INFINITY;
@@ -567,59 +693,43 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) st.o[ct] = f4{0, 0, 0, 0};
 
-    // ---- packed chunks of this wave, software-pipelined one side ahead
-    h8 qB[4];
-    {
-        int ci = c0 + wave;
-        if (ci >= c1) {
-            q_operand(qB);
-        } else {
-            KSide<BITS, GS> K;
-            VSide<BITS, GS> V;
-            const Magic mg;
-            PROF(1);
-            load_kside<BITS, GS>(K, P, bh, ci, lane);
-            load_vside<BITS, GS>(V, P, bh, ci, lane);
-            // every load of the chunk is issued before any of it is used: keep the scheduler from
-            // sinking the V loads below the QK^T work
-            __builtin_amdgcn_sched_barrier(0);
-            PROF(2);
-            q_operand(qB);
-            while (true) {
-                packed_chunk<BITS, GS, BF16>(K, V, P, bh, ci, lane, qB, lo_part, mg, st);
-                PROF(3);
-                const int cn = ci + kNW;
-                if (cn >= c1) break;
-                load_kside<BITS, GS>(K, P, bh, cn, lane);
-                load_vside<BITS, GS>(V, P, bh, cn, lane);
-                __builtin_amdgcn_sched_barrier(0);
-                ci = cn;
-            }
+    // ---- packed units of this wave
+    if (u < u1) {
+        const Magic mg;
+#ifdef BITDECODE_PROF
+        wait_vm<2>();
+        PROF(2);
+#endif
+        while (true) {
+            compute_unit<BITS, GS, BF16>(region, region_lds, A, Q, P, lane, lo_part, mg, st);
+            u += NW;
+            if (u >= u1) break;
+            A = unit_addr<BITS, GS>(P, bh, u, lane);
+            issue_first_half<BITS, GS>(A, lane, region_lds);
         }
     }
-    // ---- fp16 window tiles of this wave
+    PROF(3);
+    // ---- fp16 window tiles of this wave (the region becomes the V-transpose slab)
     {
-        uint16_t* slab = reinterpret_cast<uint16_t*>(lds_raw) + wave * kSlabHalves;
-        const int stride = kNW * P.nsplit;
+        uint16_t* slab = reinterpret_cast<uint16_t*>(region);
+        const int stride = NW * P.nsplit;
         int t = wave * P.nsplit + split;   // consecutive tiles go to different workgroups
         if (t < nT) {
+            wait_vm<0>();                  // q rows (a wave without packed units has not waited yet)
             Fp16Tile T;
             load_fp16_tile(T, P, bi, hk, t * 16, R, lane);
             while (true) {
                 const int tn = t + stride;
-                Fp16Tile N;
                 const bool more = tn < nT;
-                if (more) load_fp16_tile(N, P, bi, hk, tn * 16, R, lane);
-                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, qB, lo_part, st, slab);
+                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, Q, lo_part, st, slab);
                 if (!more) break;
-                T = N;
+                load_fp16_tile(T, P, bi, hk, tn * 16, R, lane);
                 t = tn;
             }
         }
     }
 
-    PROF(4);
-    // ---- merge the waves of this workgroup through LDS
+    // ---- merge the waves of this workgroup through LDS (each wave's slot is its own region)
     const float lsum = st.l[0] + partner(st.l[0]);      // rows are equal; lo columns hold 0
 #pragma unroll
     for (int ct = 0; ct < 8; ++ct) {
@@ -629,32 +739,32 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
             st.o[ct][r] = v + partner(v);      // hi + lo
         }
     }
-    __syncthreads();   // slabs are dead from here on
-    float* sO = reinterpret_cast<float*>(lds_raw);
     if (col < g) {
+        float* sO = reinterpret_cast<float*>(region);
 #pragma unroll
         for (int ct = 0; ct < 8; ++ct) {
-            *reinterpret_cast<f4*>(&sO[(wave * kMaxGroupHeads + col) * kHeadDim + 16 * ct + 4 * kg]) = st.o[ct];
+            *reinterpret_cast<f4*>(&sO[col * kHeadDim + 16 * ct + 4 * kg]) = st.o[ct];
         }
         if (kg == 0) {
-            sM[wave][col] = st.m * P.scale_log2;     // base-2 units
-            sL[wave][col] = lsum;
+            sM[wave * kMaxGroupHeads + col] = st.m * P.scale_log2;     // base-2 units
+            sL[wave * kMaxGroupHeads + col] = lsum;
         }
     }
     __syncthreads();
+    PROF(4);
     const int64_t hstride = static_cast<int64_t>(P.b) * P.h;       // rows per split in the workspace
-    for (int idx = tid; idx < g * kHeadDim; idx += kNW * 64) {
+    for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
         const int hh = idx >> 7, c = idx & 127;
-        float M = sM[0][hh];
+        float M = sM[hh];
 #pragma unroll
-        for (int w = 1; w < kNW; ++w) M = fmaxf(M, sM[w][hh]);
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, sM[w * kMaxGroupHeads + hh]);
         const float Mu = (M == -INFINITY) ? 0.0f : M;
         float L = 0.0f, O = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kNW; ++w) {
-            const float a = __builtin_amdgcn_exp2f(sM[w][hh] - Mu);
-            L += a * sL[w][hh];
-            O += a * sO[(w * kMaxGroupHeads + hh) * kHeadDim + c];
+        for (int w = 0; w < NW; ++w) {
+            const float a = __builtin_amdgcn_exp2f(sM[w * kMaxGroupHeads + hh] - Mu);
+            L += a * sL[w * kMaxGroupHeads + hh];
+            O += a * reinterpret_cast<const float*>(lds + w * REGION)[hh * kHeadDim + c];
         }
         const bool empty = !(L > 0.0f);
         const float o = empty ? 0.0f : O / L;
@@ -681,22 +791,23 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
     // completed (vmcnt 0) and the workgroup has met at the barrier, thread 0 takes the ticket.
     // The merging workgroup reads the partials with device-scope loads, so no cache-wide
     // write-back or invalidate is needed on either side.
-    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): this thread's partial stores are complete
+    wait_vm<0>();
     __syncthreads();
     if (tid == 0) {
         const int old = __hip_atomic_fetch_add(&P.tickets[bh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == P.nsplit - 1);
-        if (s_last) __hip_atomic_store(&P.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = (old == P.nsplit - 1);
+        *s_last = last;
+        if (last) __hip_atomic_store(&P.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     PROF(6);
-    if (!s_last) {
+    if (!*s_last) {
         PROF_FLUSH();
         return;
     }
     // every thread owns one (head, channel) and fetches the partial outputs and LSEs of up to 32
     // splits in one batch, so that the whole merge costs one memory round trip
-    for (int idx = tid; idx < g * kHeadDim; idx += kNW * 64) {
+    for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
         const int hh = idx >> 7, c = idx & 127;
         const int hq = hk * g + hh;
         const int64_t row0 = bi * P.h + hq;
@@ -736,15 +847,24 @@ __global__ __launch_bounds__(kNW * 64) void fwd_splitkv_kernel(FwdParams P) {
     PROF_FLUSH();
 }
 
+template <int BITS, int GS, bool BF16>
+hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
+    constexpr int kLds = fwd_lds_bytes<BITS, GS>();
+    static bool configured = false;      // raising the dynamic-LDS limit is idempotent
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16>), dim3(P.nsplit * P.hk * P.b),
+                       dim3(UnitCfg<BITS, GS>::NW * 64), kLds, stream, P);
+    return hipGetLastError();
+}
+
 template <int BITS, int GS>
 hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
-    dim3 grid(P.nsplit, P.hk, P.b);
-    if (P.bf16) {
-        hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, true>), grid, dim3(kNW * 64), 0, stream, P);
-    } else {
-        hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, false>), grid, dim3(kNW * 64), 0, stream, P);
-    }
-    return hipGetLastError();
+    return P.bf16 ? launch_fwd_tt<BITS, GS, true>(P, stream) : launch_fwd_tt<BITS, GS, false>(P, stream);
 }
 
 }  // namespace

@@ -42,6 +42,7 @@ struct FwdParams {
     float* lse;         // optional [b][h]
     int b, h, hk, g, nsplit;
     float scale, scale_log2;   // scale_log2 = |softmax_scale| * log2(e)
+    int xcd_remap;             // (b * hk) % 8 == 0: keep the splits of one (batch, kv-head) on one XCD
     int neg_scale;             // softmax_scale < 0: the sign is folded into q
     int bits, gs, bf16;
 };

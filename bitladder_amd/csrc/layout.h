@@ -30,6 +30,8 @@
 //   32*sb + 16*(i/4) + 4*kg + i%4, nibble p = i/2 + 4*(i%2).
 // V codes, 2-bit: chunk = 2 sub-blocks of 64 tokens, same halves/lanes/dwords; element
 //   e = 8*ks + i is token 64*sb2 + 32*ks + 16*(i/4) + 4*kg + i%4, field f = e/2 + 8*(e%2).
+// Parameters (scale, zero) are stored as fp16 bit patterns for both element types; a bf16 cache
+// stores fp16(bf16 value), which is the same number inside the fp16 normal range.
 // K params: per group of gs tokens 512 B: scale[128] then zero[128], natural channel order.
 // V params: per chunk 4 sub-blocks x ncg channel groups x 128 B: scale[q][i] (64 B) then
 //   zero[q][i] (64 B), q = 0..3, i = 0..7, token 32*sb + 16*(i/4) + 4*q + i%4.
@@ -52,5 +54,18 @@ constexpr int v_param_chunk_bytes(int gs) { return kChunk * (kHeadDim / gs) * 4;
 constexpr int64_t code_region_bytes(int64_t S, int bits) { return S * kHeadDim * bits / 8; }
 constexpr int64_t k_param_region_bytes(int64_t S, int gs) { return (S / gs) * kKParamGroupBytes; }
 constexpr int64_t v_param_region_bytes(int64_t S, int gs) { return S * (kHeadDim / gs) * 4; }
+
+// ---- decode work units (shared by the kernel and the host-side split choice)
+// A decode wave streams units of 4 KB of K codes + 4 KB of V codes + their parameters through its
+// private LDS region: 64 tokens at 4 bits, 128 tokens at 2 bits.
+constexpr int unit_tokens(int bits) { return bits == 4 ? 64 : 128; }
+constexpr int unit_region_bytes(int bits, int gs) {
+    const int ut = unit_tokens(bits);
+    const int kpb = (ut > gs ? ut / gs : 1) * kKParamGroupBytes;
+    const int vpb = ut * (kHeadDim / gs) * 4;
+    return 8192 + (kpb + vpb + 1023) / 1024 * 1024;
+}
+// waves per decode workgroup: as many as 160 KB of LDS (less shared scratch) and the register file allow
+constexpr int decode_waves(int bits, int gs) { return unit_region_bytes(bits, gs) <= 9216 ? 16 : 12; }
 
 }  // namespace bitdecode

@@ -47,6 +47,16 @@ __device__ __forceinline__ uint16_t from_f32(float f) {
     }
 }
 
+// Parameter as stored in the cache.  Scale and zero are rounded to the element type (fp16, or bf16
+// for bf16 inputs: that is the value the quantizer defines) and then written as fp16 bits in both
+// cases, because the decode kernel's MFMA operands are fp16.  For bf16 this is exact whenever the
+// value lies in the fp16 normal range, which is the domain the decode kernel supports anyway.
+template <bool BF16>
+__device__ __forceinline__ uint16_t param_bits(float v) {
+    if constexpr (BF16) v = to_f32<true>(from_f32<true>(v));
+    return from_f32<false>(v);
+}
+
 // qpack.h:243-251: scale_inv = range > 0 ? M / range : 0; stored scale = 1 / scale_inv (or 0)
 __device__ __forceinline__ void group_params(float mn, float mx, float M, float& sinv, float& scale) {
     float range = __fsub_rn(mx, mn);
@@ -134,8 +144,8 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
         k_mn[grp][c] = mn;
         uint16_t* kp = reinterpret_cast<uint16_t*>(
             P.k_params + bh * P.kparams_bh + (static_cast<int64_t>(ci) * NG + grp) * kKParamGroupBytes);
-        kp[c] = from_f32<BF16>(scale);
-        kp[kHeadDim + c] = from_f32<BF16>(mn);
+        kp[c] = param_bits<BF16>(scale);
+        kp[kHeadDim + c] = param_bits<BF16>(mn);
     }
     __syncthreads();
     {
@@ -227,8 +237,8 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
             v_sinv[n][cg] = sinv;
             v_mn[n][cg] = pmn[pt];
             uint16_t* dst = reinterpret_cast<uint16_t*>(vp + (sb * NCG + cg) * 128 + q * 16 + i * 2);
-            dst[0] = from_f32<BF16>(scale);
-            dst[32] = from_f32<BF16>(pmn[pt]);   // zeros start 64 bytes after the scales
+            dst[0] = param_bits<BF16>(scale);
+            dst[32] = param_bits<BF16>(pmn[pt]);   // zeros start 64 bytes after the scales
         }
     }
     __syncthreads();

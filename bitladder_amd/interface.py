@@ -266,7 +266,7 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
     with torch.cuda.device(device):
         ns = int(num_splits)
         if ns == 0:
-            ns = L.bitdecode_num_splits(b, h_k, a.max_seqlen_k, a.max_res_len, 0)
+            ns = L.bitdecode_num_splits(b, h_k, a.max_seqlen_k, a.max_res_len, 0, num_bits, group_size)
         a.num_splits = ns
         nbytes = L.bitdecode_fwd_workspace_bytes(b, h, ns)
         if nbytes:

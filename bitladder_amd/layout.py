@@ -97,11 +97,27 @@ def _dwords_to_codes(dwords: np.ndarray, tok_f, ch_f, bits: int) -> np.ndarray:
     return out
 
 
-def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int, gs: int):
-    """Logical -> physical.  codes uint8 [b,S,h,128]; k_scale/k_zero uint16 bit patterns
-    [b,S/gs,h,128]; v_scale/v_zero uint16 [b,S,h,128/gs].  Returns the four cache tensors as
-    numpy arrays with the reference shapes (k_pack/v_pack uint16, k_params/v_params float32
-    containers)."""
+def _bf16_bits_to_fp16_bits(x: np.ndarray) -> np.ndarray:
+    f = (x.astype(np.uint32) << 16).view(np.float32)
+    with np.errstate(over="ignore"):
+        return f.astype(np.float16).view(np.uint16)
+
+
+def _fp16_bits_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    # round to nearest even; exact when the fp16 value came from a bf16 inside the fp16 normal range
+    u = np.ascontiguousarray(x).view(np.float16).astype(np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int, gs: int, dtype: str = "fp16"):
+    """Logical -> physical.  codes uint8 [b,S,h,128]; k_scale/k_zero uint16 bit patterns of the
+    element type `dtype` [b,S/gs,h,128]; v_scale/v_zero uint16 [b,S,h,128/gs].  Returns the four
+    cache tensors as numpy arrays with the reference shapes (k_pack/v_pack uint16,
+    k_params/v_params float32 containers).  Parameters are stored as fp16 bits for both element
+    types (bf16 values are converted, exact inside the fp16 normal range)."""
+    if dtype == "bf16":
+        k_scale, k_zero, v_scale, v_zero = (_bf16_bits_to_fp16_bits(np.ascontiguousarray(a))
+                                            for a in (k_scale, k_zero, v_scale, v_zero))
     b, S, h, d = k_codes.shape
     assert d == D and S % CHUNK == 0
     nc, pn, ncg = S // CHUNK, 16 // bits, D // gs
@@ -126,10 +142,10 @@ def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int,
     return k_pack, k_params, v_pack, v_params
 
 
-def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int):
+def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int, dtype: str = "fp16"):
     """Physical -> logical; inverse of pack_physical.  Inputs are numpy arrays with the reference
     shapes (any 16-bit / 32-bit dtype).  Returns (k_codes, k_scale, k_zero, v_codes, v_scale,
-    v_zero) with scale/zero as uint16 bit patterns."""
+    v_zero) with scale/zero as uint16 bit patterns of the element type `dtype`."""
     b, S, h, dp = v_pack.shape
     pn = 16 // bits
     d = dp * pn
@@ -153,4 +169,6 @@ def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int):
     vz[..., tokmap] = vp[:, :, :, :, :, 1].transpose(0, 1, 2, 4, 3, 5, 6)
     v_scale = np.ascontiguousarray(vs.transpose(0, 2, 4, 1, 3)).reshape(b, S, h, ncg)
     v_zero = np.ascontiguousarray(vz.transpose(0, 2, 4, 1, 3)).reshape(b, S, h, ncg)
+    if dtype == "bf16":
+        k_scale, k_zero, v_scale, v_zero = (_fp16_bits_to_bf16_bits(a) for a in (k_scale, k_zero, v_scale, v_zero))
     return k_codes, k_scale, k_zero, v_codes, v_scale, v_zero

@@ -95,9 +95,9 @@ int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
 
 /* Split count the library would choose for this problem (host function, no GPU work);
  * replaces num_splits_heuristic (csrc/bit_decode/decode_api.cpp:234-268), retuned for 256 CUs.
- * num_cus <= 0 queries the current device. */
+ * num_cus <= 0 queries the current device; returns -1 for an unsupported (bits, group_size). */
 int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
-                         int32_t num_cus);
+                         int32_t num_cus, int32_t bits, int32_t group_size);
 
 /* Workspace the split path needs: arrival counters, fp32 partial outputs and LSEs
  * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,

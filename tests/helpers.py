@@ -57,16 +57,25 @@ def oracle_physical(qkv: O.QuantKV):
     dt = qkv.dtype
     return L.pack_physical(qkv.k_codes, bits16(qkv.k_scale, dt), bits16(qkv.k_zero, dt),
                            qkv.v_codes, bits16(qkv.v_scale, dt), bits16(qkv.v_zero, dt),
-                           qkv.bits, qkv.group_size)
+                           qkv.bits, qkv.group_size, dt)
 
 
 def assert_cache_equals_oracle(cache_np, qkv: O.QuantKV):
+    """Bit-exact comparison of a packed cache with the quantizer oracle.  Codes are compared as
+    codes; scale and zero are compared as the fp16 bit patterns the cache stores (for a bf16 cache:
+    the oracle's bf16 value converted to fp16 with round-to-nearest-even, which is the identity
+    inside the fp16 normal range)."""
     from bitladder_amd import layout as L
     dt = qkv.dtype
-    kc, ks, kz, vc, vs, vz = L.unpack_physical(*cache_np, qkv.bits, qkv.group_size)
+    kc, ks, kz, vc, vs, vz = L.unpack_physical(*cache_np, qkv.bits, qkv.group_size, "fp16")
     np.testing.assert_array_equal(kc, qkv.k_codes, err_msg="K codes")
     np.testing.assert_array_equal(vc, qkv.v_codes, err_msg="V codes")
-    np.testing.assert_array_equal(ks, bits16(qkv.k_scale, dt), err_msg="K scale")
-    np.testing.assert_array_equal(kz, bits16(qkv.k_zero, dt), err_msg="K zero")
-    np.testing.assert_array_equal(vs, bits16(qkv.v_scale, dt), err_msg="V scale")
-    np.testing.assert_array_equal(vz, bits16(qkv.v_zero, dt), err_msg="V zero")
+
+    def stored(x):
+        b = bits16(x, dt)
+        return L._bf16_bits_to_fp16_bits(b) if dt == "bf16" else b
+
+    np.testing.assert_array_equal(ks, stored(qkv.k_scale), err_msg="K scale")
+    np.testing.assert_array_equal(kz, stored(qkv.k_zero), err_msg="K zero")
+    np.testing.assert_array_equal(vs, stored(qkv.v_scale), err_msg="V scale")
+    np.testing.assert_array_equal(vz, stored(qkv.v_zero), err_msg="V zero")

@@ -36,6 +36,24 @@ def test_layout_roundtrip_and_byte_budget(bits, gs):
         np.testing.assert_array_equal(a, c)
 
 
+def test_bf16_parameters_are_stored_as_fp16_bits():
+    """A bf16 cache keeps scale/zero as fp16 bit patterns: bf16 values inside the fp16 normal range
+    survive pack -> unpack unchanged, and the stored pattern is the fp16 encoding of the value."""
+    rng = np.random.default_rng(5)
+    b, S, h, bits, gs = 1, 128, 2, 4, 64
+    kc = rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8)
+    vals = rng.choice(np.array([1.0, -2.5, 0.0078125, 1000.0, -6.4849853515625e-05, 65280.0], np.float32), (b, S // gs, h, 128))
+    as_bf16 = (vals.view(np.uint32) >> 16).astype(np.uint16)            # all exactly representable in bf16
+    vsz = np.full((b, S, h, 128 // gs), 0x3F80, np.uint16)              # bf16 1.0
+    phys = L.pack_physical(kc, as_bf16, as_bf16, kc, vsz, vsz, bits, gs, "bf16")
+    stored = np.ascontiguousarray(phys[1]).reshape(-1).view(np.float16).reshape(b, h, S // gs, 2, 128)
+    np.testing.assert_array_equal(stored[:, :, :, 0].transpose(0, 2, 1, 3).astype(np.float32), vals)
+    assert np.ascontiguousarray(phys[3]).reshape(-1).view(np.uint16)[0] == 0x3C00   # fp16 1.0
+    back = L.unpack_physical(*phys, bits, gs, "bf16")
+    np.testing.assert_array_equal(back[1], as_bf16)
+    np.testing.assert_array_equal(back[4], vsz)
+
+
 @pytest.mark.parametrize("bits", [2, 4])
 def test_code_maps_are_bijections_and_chunk_local(bits):
     for fn in (L.k_code_map, L.v_code_map):
@@ -183,13 +201,15 @@ def test_qpack_of_zero_tokens_is_a_no_op():
 
 def test_split_choice_and_workspace_size():
     lib = _lib.lib()
-    # 32K GQA config on 256 CUs: 8 kv heads x 32 splits = one workgroup per CU, one chunk per wave
-    assert lib.bitdecode_num_splits(1, 8, 32768, 128, 256) == 32
+    # 32K GQA config on 256 CUs: 8 kv heads x 32 splits = one workgroup per CU, one 64-token unit per wave
+    assert lib.bitdecode_num_splits(1, 8, 32768, 128, 256, 4, 128) == 32
     # enough (batch x kv-head) workgroups already: no split
-    assert lib.bitdecode_num_splits(64, 8, 4096, 128, 256) == 1
-    # never more splits than there is work for
-    assert lib.bitdecode_num_splits(1, 1, 256, 0, 256) == 1
-    assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256) == 3
+    assert lib.bitdecode_num_splits(64, 8, 4096, 128, 256, 4, 128) == 1
+    # never more splits than there is work for: 4 units of 64 tokens -> one workgroup
+    assert lib.bitdecode_num_splits(1, 1, 256, 0, 256, 4, 128) == 1
+    # 48 units over 16 waves -> 3 splits
+    assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256, 4, 128) == 3
+    assert lib.bitdecode_num_splits(1, 1, 1024, 0, 256, 3, 128) == -1
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 256 + 32 * 32 * 129 * 4
 
