@@ -79,12 +79,12 @@ int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t m
     return choose_splits(b, h_k, max_seqlen_k, max_res_len, num_cus, bits, group_size);
 }
 
-// [tickets: b*h ints rounded up to 256 B][o_part][lse_part]
+// [tickets: b*h ints rounded up to 256 B][o_part][ml_part]
 static size_t ticket_bytes(int32_t b, int32_t h) { return (static_cast<size_t>(b) * h * sizeof(int) + 255) / 256 * 256; }
 
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     if (num_splits <= 1) return 0;
-    return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 1) * sizeof(float);
+    return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 2) * sizeof(float);
 }
 
 int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
@@ -165,6 +165,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
 
     int nsplit = a->num_splits;
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
+    if (nsplit > 512) return fail(BITDECODE_EINVAL, "num_splits %d is above the limit of 512", nsplit);
     if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
     if (nsplit > 1) {
         const size_t need = bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
@@ -203,7 +204,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     if (nsplit > 1) {
         P.tickets = static_cast<int*>(a->workspace);
         P.o_part = reinterpret_cast<float*>(static_cast<uint8_t*>(a->workspace) + ticket_bytes(a->b, a->h));
-        P.lse_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
+        P.ml_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
     }
     hipError_t e = launch_fwd(P, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));

@@ -52,7 +52,7 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 // Optional per-wave timeline for kernel tuning (built only with -DBITDECODE_PROF).
 #ifdef BITDECODE_PROF
 __device__ unsigned long long* g_prof = nullptr;
-#define PROF_DECL unsigned long long prof_ts[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define PROF_DECL unsigned long long prof_ts[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
 #define PROF(slot)                                 \
     do {                                           \
         __builtin_amdgcn_sched_barrier(0);         \
@@ -63,11 +63,20 @@ __device__ unsigned long long* g_prof = nullptr;
     do {                                                                                              \
         unsigned long long* pb = g_prof;                                                              \
         if (pb && (threadIdx.x & 63) == 0) {                                                          \
-            pb += ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 8;                                  \
-            for (int i_ = 0; i_ < 8; ++i_) pb[i_] = prof_ts[i_];                                      \
+            pb += ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16;                                 \
+            for (int i_ = 0; i_ < 16; ++i_) pb[i_] = prof_ts[i_];                                     \
         }                                                                                             \
     } while (0)
+#define PHASE(slot)                                                 \
+    do {                                                            \
+        if (phase_ts) {                                             \
+            __builtin_amdgcn_sched_barrier(0);                      \
+            phase_ts[slot] = __builtin_readcyclecounter();          \
+            __builtin_amdgcn_sched_barrier(0);                      \
+        }                                                           \
+    } while (0)
 #else
+#define PHASE(slot) do { } while (0)
 #define PROF_DECL do { } while (0)
 #define PROF(slot) do { } while (0)
 #define PROF_FLUSH() do { } while (0)
@@ -233,9 +242,10 @@ template <int BITS, int GS>
 struct UnitCfg {
     static constexpr int UT = unit_tokens(BITS);             // tokens per unit (4 KB of K codes, 4 KB of V codes)
     static constexpr int UPC = kChunk / UT;                  // units per 128-token chunk
-    static constexpr int NTILE = UT / 16;                    // 16-token tiles per unit
-    static constexpr int TPS = NTILE / 2;                    // tiles per step (two steps per unit)
-    static constexpr int NKS = TPS / 2;                      // 32-token k-steps (V sub-blocks) per step
+    static constexpr int NSTEP = UT / 64;                    // 64-token steps per unit (one softmax pass each)
+    static constexpr int TPS = 4;                            // 16-token tiles per step
+    static constexpr int NKS = 2;                            // 32-token k-steps (V sub-blocks) per step
+    static constexpr int RPS = 4 / NSTEP;                    // 1 KB rows of K codes (and of V codes) per step
     static constexpr int TPG = GS / 16;                      // tiles per K group
     static constexpr int NGU = UT > GS ? UT / GS : 1;        // K groups a unit touches
     static constexpr int NCG = kHeadDim / GS;                // V channel groups
@@ -295,10 +305,11 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
         (const __attribute__((address_space(3))) void*)p));
 }
 
-// The loads of unit u, in the order they are consumed.  First half: params, K rows 0-1, V rows 0-1
-// (step 0); second half: K rows 2-3, V rows 2-3 (step 1).  The second half is issued while step 0
-// is being computed: a wave stalls while the memory pipeline will not take its next load, so it
-// only queues what it needs next and keeps the VALU busy in between.
+// The loads of unit u, in the order they are consumed: the parameter rows, then per 64-token step
+// its K rows and its V rows.  The first unit of a wave is issued in one go; for later units of a
+// two-step unit the second step is issued while the first is being computed (a wave stalls while
+// the memory pipeline will not take its next load, so it queues what it needs next and keeps the
+// VALU busy in between).
 template <int BITS, int GS>
 struct UnitAddr {
     const uint8_t* kc;
@@ -319,7 +330,7 @@ __device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int6
     return A;
 }
 template <int BITS, int GS>
-__device__ __forceinline__ void issue_first_half(const UnitAddr<BITS, GS>& A, int lane, uint32_t region) {
+__device__ __forceinline__ void issue_params(const UnitAddr<BITS, GS>& A, int lane, uint32_t region) {
     using C = UnitCfg<BITS, GS>;
 #pragma unroll
     for (int r = 0; r < C::PROWS; ++r) {
@@ -328,17 +339,28 @@ __device__ __forceinline__ void issue_first_half(const UnitAddr<BITS, GS>& A, in
             o < C::KPB ? A.kp + o : (o < C::KPB + C::VPB ? A.vp + (o - C::KPB) : A.kp + (o & (C::KPB - 1)));
         dma_row(src, region + 8192 + r * 1024);
     }
-    dma_row(A.kc, region);
-    dma_row(A.kc + 1024, region + 1024);
-    dma_row(A.vc, region + 4096);
-    dma_row(A.vc + 1024, region + 4096 + 1024);
 }
 template <int BITS, int GS>
-__device__ __forceinline__ void issue_second_half(const UnitAddr<BITS, GS>& A, uint32_t region) {
-    dma_row(A.kc + 2048, region + 2048);
-    dma_row(A.kc + 3072, region + 3072);
-    dma_row(A.vc + 2048, region + 4096 + 2048);
-    dma_row(A.vc + 3072, region + 4096 + 3072);
+__device__ __forceinline__ void issue_step(const UnitAddr<BITS, GS>& A, uint32_t region, int step) {
+    using C = UnitCfg<BITS, GS>;
+#pragma unroll
+    for (int r = 0; r < C::RPS; ++r) dma_row(A.kc + (step * C::RPS + r) * 1024, region + (step * C::RPS + r) * 1024);
+#pragma unroll
+    for (int r = 0; r < C::RPS; ++r) {
+        dma_row(A.vc + (step * C::RPS + r) * 1024, region + 4096 + (step * C::RPS + r) * 1024);
+    }
+}
+// FULL: params and every step; otherwise params and step 0 (compute_unit issues the rest)
+template <int BITS, int GS, bool FULL>
+__device__ __forceinline__ void issue_unit(const UnitAddr<BITS, GS>& A, int lane, uint32_t region) {
+    issue_params<BITS, GS>(A, lane, region);
+    issue_step<BITS, GS>(A, region, 0);
+    if (FULL && UnitCfg<BITS, GS>::NSTEP > 1) issue_step<BITS, GS>(A, region, 1);
+}
+template <int BITS, int GS, bool FULL>
+constexpr int unit_loads() {
+    using C = UnitCfg<BITS, GS>;
+    return C::PROWS + 2 * C::RPS * (FULL ? C::NSTEP : 1);
 }
 
 // Per-group state of the K side: Q with the group's scale folded in (exact hi/lo split) and the
@@ -357,9 +379,12 @@ struct QRows {
     const uint8_t* qz;   // same row in the hi columns, zero row in the lo columns
     const uint8_t* qm;   // zero row in the hi columns, same row in the lo columns
 };
+// Rows are 272 bytes apart (256 + 16 of padding) so that the eight heads read by neighbouring
+// lanes fall into different LDS banks.
+constexpr int kQRowBytes = 272;
 __device__ __forceinline__ QRows q_rows(const uint8_t* sq, int head, int kg, bool lo_part) {
-    const uint8_t* row = sq + head * 256 + kg * 16;
-    const uint8_t* zero = sq + 8 * 256 + kg * 16;
+    const uint8_t* row = sq + head * kQRowBytes + kg * 16;
+    const uint8_t* zero = sq + 8 * kQRowBytes + kg * 16;
     return QRows{row, lo_part ? zero : row, lo_part ? row : zero};
 }
 __device__ __forceinline__ h8 q_load(const uint8_t* row, int j) {
@@ -387,36 +412,48 @@ __device__ __forceinline__ void start_group(KGroup& G, const uint8_t* kpar, cons
     }
 }
 
-// One packed unit from the wave's LDS region, in two steps: S^T tiles of the step, online
+// One packed unit from the wave's LDS region, in 64-token steps: S^T tiles of the step, online
 // softmax update, O^T += V^T P^T for the same tokens.  Scores stay in q.k units; the softmax
-// scale is applied inside the exponent.  `pending` = loads issued after this unit's (0 here).
-template <int BITS, int GS, bool BF16>
+// scale is applied inside the exponent.  FULL: all loads of the unit are already in flight.
+template <int BITS, int GS, bool BF16, bool FULL>
 __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, const UnitAddr<BITS, GS>& A,
                                              const QRows& Q, const FwdParams& P, int lane, bool lo_part,
-                                             const Magic& mg, WaveState<kHeadDim / GS>& st) {
+                                             const Magic& mg, WaveState<kHeadDim / GS>& st,
+                                             unsigned long long* phase_ts = nullptr) {
     using C = UnitCfg<BITS, GS>;
     constexpr int NCG = C::NCG, TPS = C::TPS, NKS = C::NKS, TPG = C::TPG, CTPG = GS / 16;
+    constexpr int NSTEP = C::NSTEP, RPS = C::RPS, STEP_LOADS = 2 * RPS;
     const int kg = lane >> 4;
     const h8 noff = -code_offsets<BITS>();
     const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
-    const bool neg = P.neg_scale != 0;
     const uint32_t hi_cols = lo_part ? 0u : 0xffffffffu;
     const u4* kcode = reinterpret_cast<const u4*>(reg) + lane;             // row r: kcode[64 * r]
     const u4* vcode = reinterpret_cast<const u4*>(reg + 4096) + lane;
     const uint8_t* kpar = reg + 8192;
     const uint8_t* vpar = reg + 8192 + C::KPB + kg * 16;
 
+    // the parameter rows lead the queue: the first K group is prepared while the code rows arrive
+    wait_vm<STEP_LOADS * (FULL ? NSTEP : 1)>();
+    PHASE(8);
     KGroup G;
+    start_group<BITS, BF16>(G, kpar, Q, kg);
+    (void)phase_ts;
 #pragma unroll
-    for (int step = 0; step < 2; ++step) {
-        // loads still allowed in flight when the K rows of this step are needed: its two V rows
-        wait_vm<2>();
+    for (int step = 0; step < NSTEP; ++step) {
+        // loads allowed in flight when the K rows of this step are needed: its V rows and later steps
+        constexpr int kLaterFull = STEP_LOADS * (NSTEP - 1);
+        if (step == 0) {
+            if (FULL) wait_vm<RPS + kLaterFull>(); else wait_vm<RPS>();
+        } else {
+            wait_vm<RPS>();
+        }
+        PHASE(9 + 3 * step);
         float t[4 * TPS];
 #pragma unroll
         for (int tt = 0; tt < TPS; ++tt) {
             const int tile = step * TPS + tt;
-            if (tile == 0 || tile % TPG == 0) {
-                start_group<BITS, BF16>(G, kpar + ((tile * 16) / GS) * kKParamGroupBytes * (C::NGU > 1 ? 1 : 0), Q, kg);
+            if (tile != 0 && tile % TPG == 0) {
+                start_group<BITS, BF16>(G, kpar + ((tile * 16) / GS) * kKParamGroupBytes, Q, kg);
             }
             f4 acc = G.kb;
             if constexpr (BITS == 4) {
@@ -436,11 +473,8 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
 #pragma unroll
             for (int r = 0; r < 4; ++r) t[4 * tt + r] = acc[r] + partner(acc[r]);   // hi + lo
         }
-        if (step == 0) issue_second_half<BITS, GS>(A, region_lds);
-        if (neg) {      // softmax_scale < 0: scale_log2 holds |scale|, the sign goes into the scores
-#pragma unroll
-            for (int i = 0; i < 4 * TPS; ++i) t[i] = -t[i];
-        }
+        if (!FULL && step + 1 < NSTEP) issue_step<BITS, GS>(A, region_lds, step + 1);
+        PHASE(10 + 3 * step);
 
         softmax_step<4 * TPS, NCG>(t, P.scale_log2, st);
 
@@ -458,8 +492,8 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
             pm[ks] = __builtin_bit_cast(h8, pw & ~hi_cols);      // and only in the lo columns
             st.l = mfma32(ones, pz[ks], st.l);
         }
-        if (step == 0) wait_vm<4>(); else wait_vm<0>();
-        const u4 w0 = vcode[64 * (2 * step)], w1 = vcode[64 * (2 * step + 1)];
+        PHASE(11 + 3 * step);
+        if (step + 1 < NSTEP) wait_vm<STEP_LOADS>(); else wait_vm<0>();
 #pragma unroll
         for (int cg = 0; cg < NCG; ++cg) {
             h8 pp[NKS];
@@ -475,18 +509,24 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
 #pragma unroll
             for (int x = 0; x < CTPG; ++x) {
                 const int ct = cg * CTPG + x;
-                const uint32_t w = ct < 4 ? w0[ct & 3] : w1[ct & 3];
                 if constexpr (BITS == 4) {
-                    st.o[ct] = mfma32(dq4(w, mg), pp[0], st.o[ct]);
+                    // rows of the step: (sub-block ks, channel half ct / 4)
+#pragma unroll
+                    for (int ks = 0; ks < NKS; ++ks) {
+                        const uint32_t w = vcode[64 * (2 * ks + ct / 4)][ct & 3];
+                        st.o[ct] = mfma32(dq4(w, mg), pp[ks], st.o[ct]);
+                    }
                 } else {
+                    const uint32_t w = vcode[64 * (2 * step + ct / 4)][ct & 3];
                     h8 a0, a1;
                     dq2(w, a0, a1, mg);
                     st.o[ct] = mfma32(a0, pp[0], st.o[ct]);
-                    st.o[ct] = mfma32(a1, pp[NKS - 1], st.o[ct]);
+                    st.o[ct] = mfma32(a1, pp[1], st.o[ct]);
                 }
             }
         }
     }
+    PHASE(15);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -542,7 +582,6 @@ __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P,
         for (int r = 0; r < 4; ++r) {
             const int tk = n0 + 4 * kg + r;
             float tot = acc[r] + partner(acc[r]);   // outside the select: every lane executes the DPP
-            if (P.neg_scale) tot = -tot;
             s[r] = tk < R ? tot : -INFINITY;
         }
     }
@@ -579,6 +618,40 @@ __device__ __forceinline__ float ld_dev(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// partial outputs of splits s0 .. s0+31 (clamped to the last split) for one (head, channel)
+__device__ __forceinline__ void load_partials(float (&v)[32], const float* o_part, int64_t item, int64_t split_stride,
+                                              int s0, int nsplit) {
+    const float* p = o_part + s0 * split_stride + item;
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+        v[k] = ld_dev(p);
+        if (s0 + k + 1 < nsplit) p += split_stride;
+    }
+}
+// (maximum, sum) pairs of splits s0 + s8 + 8k, k = 0..7 (clamped to the last split), for one head
+__device__ __forceinline__ void load_ml(float (&m)[8], float (&l)[8], const float* ml_part, int64_t row,
+                                        int64_t split_stride, int s0, int s8, int nsplit) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int sp = min(s0 + s8 + 8 * k, nsplit - 1);
+        const float* src = ml_part + 2 * (sp * split_stride + row);
+        m[k] = ld_dev(src);
+        l[k] = ld_dev(src + 1);
+    }
+}
+
+// reductions over the eight lanes that share lane % 8 (one head), in a fixed butterfly order
+__device__ __forceinline__ float head_max(float x) {
+    x = fmaxf(x, __shfl_xor(x, 8));
+    x = fmaxf(x, __shfl_xor(x, 16));
+    return fmaxf(x, __shfl_xor(x, 32));
+}
+__device__ __forceinline__ float head_sum(float x) {
+    x += __shfl_xor(x, 8);
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
+}
+
 template <bool BF16>
 __device__ __forceinline__ uint16_t to_out(float f) {
     if constexpr (BF16) {
@@ -606,7 +679,7 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 template <int BITS, int GS>
 constexpr int fwd_lds_bytes() {
     using C = UnitCfg<BITS, GS>;
-    return C::NW * C::REGION + (kMaxGroupHeads + 1) * 256 + 2 * C::NW * kMaxGroupHeads * 4 + 16;
+    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + (3 * C::NW + 2) * kMaxGroupHeads * 4 + 16;
 }
 
 template <int BITS, int GS, bool BF16>
@@ -615,9 +688,11 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t* const sq = lds + NW * REGION;                                   // [8 + zero row][128] 16-bit q
-    float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * 256);   // [NW][8]
+    float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * kQRowBytes);   // [NW][8]
     float* const sL = sM + NW * kMaxGroupHeads;
-    int* const s_last = reinterpret_cast<int*>(sL + NW * kMaxGroupHeads);
+    float* const sA = sL + NW * kMaxGroupHeads;                                   // [8][NW] merge weights
+    float* const sHead = sA + NW * kMaxGroupHeads;                                // [2][8] merged max, sum
+    int* const s_last = reinterpret_cast<int*>(sHead + 2 * kMaxGroupHeads);
 
     PROF_DECL;
     PROF(0);
@@ -673,14 +748,24 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     UnitAddr<BITS, GS> A;
     if (u < u1) {
         A = unit_addr<BITS, GS>(P, bh, u, lane);
-        issue_first_half<BITS, GS>(A, lane, region_lds);
-        wait_then_take<C::PROWS + 4>(qa, qb, qa_raw, qb_raw);
+        issue_unit<BITS, GS, true>(A, lane, region_lds);
+        wait_then_take<unit_loads<BITS, GS, true>()>(qa, qb, qa_raw, qb_raw);
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
     }
-    *reinterpret_cast<h8*>(sq + lane * 16) = cvt_h8<BF16>(qa);
-    *reinterpret_cast<h8*>(sq + 1024 + lane * 16) = cvt_h8<BF16>(qb);
-    if (lane < 16) *reinterpret_cast<u4*>(sq + 8 * 256 + lane * 16) = u4{0, 0, 0, 0};
+    if (P.neg_scale) {      // softmax_scale < 0: scale_log2 holds |scale|, the sign goes into q
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            qa[i] ^= 0x80008000u;
+            qb[i] ^= 0x80008000u;
+        }
+    }
+    {
+        uint8_t* dst = sq + (lane >> 4) * kQRowBytes + (lane & 15) * 16;
+        *reinterpret_cast<h8*>(dst) = cvt_h8<BF16>(qa);
+        *reinterpret_cast<h8*>(dst + 4 * kQRowBytes) = cvt_h8<BF16>(qb);
+        if (lane < 16) *reinterpret_cast<u4*>(sq + 8 * kQRowBytes + lane * 16) = u4{0, 0, 0, 0};
+    }
     // (head slots past the group hold head 0 again: finite values whose results are never stored)
     const QRows Q = q_rows(sq, head, kg, lo_part);
     PROF(1);
@@ -697,15 +782,18 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     if (u < u1) {
         const Magic mg;
 #ifdef BITDECODE_PROF
-        wait_vm<2>();
+        wait_vm<2 * C::RPS * C::NSTEP>();   // parameter rows have arrived
         PROF(2);
 #endif
-        while (true) {
-            compute_unit<BITS, GS, BF16>(region, region_lds, A, Q, P, lane, lo_part, mg, st);
-            u += NW;
-            if (u >= u1) break;
+#ifdef BITDECODE_PROF
+        compute_unit<BITS, GS, BF16, true>(region, region_lds, A, Q, P, lane, lo_part, mg, st, prof_ts);
+#else
+        compute_unit<BITS, GS, BF16, true>(region, region_lds, A, Q, P, lane, lo_part, mg, st);
+#endif
+        for (u += NW; u < u1; u += NW) {
             A = unit_addr<BITS, GS>(P, bh, u, lane);
-            issue_first_half<BITS, GS>(A, lane, region_lds);
+            issue_unit<BITS, GS, false>(A, lane, region_lds);
+            compute_unit<BITS, GS, BF16, false>(region, region_lds, A, Q, P, lane, lo_part, mg, st);
         }
     }
     PROF(3);
@@ -745,39 +833,67 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         for (int ct = 0; ct < 8; ++ct) {
             *reinterpret_cast<f4*>(&sO[col * kHeadDim + 16 * ct + 4 * kg]) = st.o[ct];
         }
-        if (kg == 0) {
-            sM[wave * kMaxGroupHeads + col] = st.m * P.scale_log2;     // base-2 units
-            sL[wave * kMaxGroupHeads + col] = lsum;
-        }
+    }
+    if (kg == 0 && col < kMaxGroupHeads) {
+        sM[wave * kMaxGroupHeads + col] = col < g ? st.m * P.scale_log2 : -INFINITY;     // base-2 units
+        sL[wave * kMaxGroupHeads + col] = col < g ? lsum : 0.0f;
     }
     __syncthreads();
     PROF(4);
+    // one wave turns the per-wave maxima and sums into weights: lane (w8, head) covers waves w8, w8 + 8
+    if (wave == 0) {
+        const int hh = lane & 7, w8 = lane >> 3;
+        const bool two = w8 + 8 < NW;
+        const float m0 = sM[w8 * kMaxGroupHeads + hh];
+        const float m1 = two ? sM[(w8 + 8) * kMaxGroupHeads + hh] : -INFINITY;
+        const float M = head_max(fmaxf(m0, m1));
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        const float a0 = __builtin_amdgcn_exp2f(m0 - Mu), a1 = __builtin_amdgcn_exp2f(m1 - Mu);
+        sA[hh * NW + w8] = a0;
+        float L = a0 * sL[w8 * kMaxGroupHeads + hh];
+        if (two) {
+            sA[hh * NW + w8 + 8] = a1;
+            L += a1 * sL[(w8 + 8) * kMaxGroupHeads + hh];
+        }
+        L = head_sum(L);
+        if (w8 == 0) {
+            sHead[hh] = M;
+            sHead[kMaxGroupHeads + hh] = L;
+        }
+    }
+    __syncthreads();
+    // the workgroup's result relative to its own maximum: O = sum_w a_w O_w, with (M, L) per head.
+    // A single split normalises and writes the output; otherwise the triple is published as is.
     const int64_t hstride = static_cast<int64_t>(P.b) * P.h;       // rows per split in the workspace
     for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
         const int hh = idx >> 7, c = idx & 127;
-        float M = sM[hh];
+        float aw[NW];      // NW is a multiple of 4: four weights per LDS read
 #pragma unroll
-        for (int w = 1; w < NW; ++w) M = fmaxf(M, sM[w * kMaxGroupHeads + hh]);
-        const float Mu = (M == -INFINITY) ? 0.0f : M;
-        float L = 0.0f, O = 0.0f;
+        for (int w = 0; w < NW; w += 4) {
+            const f4 a4 = *reinterpret_cast<const f4*>(&sA[hh * NW + w]);
+            aw[w] = a4[0]; aw[w + 1] = a4[1]; aw[w + 2] = a4[2]; aw[w + 3] = a4[3];
+        }
+        float O = 0.0f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            const float a = __builtin_amdgcn_exp2f(sM[w * kMaxGroupHeads + hh] - Mu);
-            L += a * sL[w * kMaxGroupHeads + hh];
-            O += a * reinterpret_cast<const float*>(lds + w * REGION)[hh * kHeadDim + c];
+            O += aw[w] * reinterpret_cast<const float*>(lds + w * REGION)[hh * kHeadDim + c];
         }
-        const bool empty = !(L > 0.0f);
-        const float o = empty ? 0.0f : O / L;
-        // natural-log LSE of this split (softmax.h:303); -inf marks an empty split
-        const float lse = empty ? -INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+        const float M = sHead[hh], L = sHead[kMaxGroupHeads + hh];
         const int hq = hk * g + hh;
         if (P.nsplit == 1) {
-            P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(o);
-            if (c == 0 && P.lse) P.lse[bi * P.h + hq] = empty ? INFINITY : lse;
+            const bool empty = !(L > 0.0f);
+            P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(empty ? 0.0f : O / L);
+            // natural-log LSE (softmax.h:303); +inf for a row without keys
+            if (c == 0 && P.lse) {
+                P.lse[bi * P.h + hq] = empty ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+            }
         } else {
             const int64_t row = split * hstride + bi * P.h + hq;
-            st_dev(&P.o_part[row * kHeadDim + c], o);
-            if (c == 0) st_dev(&P.lse_part[row], lse);
+            st_dev(&P.o_part[row * kHeadDim + c], O);
+            if (c == 0) {
+                st_dev(&P.ml_part[2 * row], M);
+                st_dev(&P.ml_part[2 * row + 1], L);
+            }
         }
     }
     PROF(5);
@@ -805,43 +921,82 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         PROF_FLUSH();
         return;
     }
-    // every thread owns one (head, channel) and fetches the partial outputs and LSEs of up to 32
-    // splits in one batch, so that the whole merge costs one memory round trip
+    // Every thread owns one (head, channel) and starts fetching the partial outputs of the first 32
+    // splits at once; meanwhile wave 0 fetches the (M, L) pairs, lane (s8, head) taking splits
+    // s8, s8 + 8, ..., and turns them into one weight per split and head in LDS (the regions are
+    // free by now).  out = sum_s w_s O_s / sum_s w_s L_s.
+    const int nsp32 = (P.nsplit + 31) & ~31;
+    float* const tM = reinterpret_cast<float*>(lds);                  // [nsplit][8] maxima
+    float* const tL = tM + P.nsplit * kMaxGroupHeads;                  // [nsplit][8] sums
+    float* const sW = tL + P.nsplit * kMaxGroupHeads;                  // [8][nsp32] weights, zero past nsplit
+    const int64_t row00 = bi * P.h + hk * g;
+    float v0[32], m8[8], l8[8];
+    const int wl_hh = lane & 7, wl_s8 = lane >> 3;
+    const int64_t wl_row = row00 + (wl_hh < g ? wl_hh : 0);
+    if (wave == 0) load_ml(m8, l8, P.ml_part, wl_row, hstride, 0, wl_s8, P.nsplit);     // ahead of the bulk loads
+    if (tid < g * kHeadDim) load_partials(v0, P.o_part, (row00 + (tid >> 7)) * kHeadDim + (tid & 127),
+                                          hstride * kHeadDim, 0, P.nsplit);
+    PROF(12);
+    if (wave == 0) {
+        const int hh = wl_hh, s8 = wl_s8;
+        const bool live = hh < g;
+        float M = -INFINITY;
+        for (int sb = 0; sb < P.nsplit; sb += 64) {      // eight splits per lane and round
+            if (sb > 0) load_ml(m8, l8, P.ml_part, wl_row, hstride, sb, s8, P.nsplit);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int sp = sb + s8 + 8 * k;
+                if (sp < P.nsplit) {
+                    const float mk = live ? m8[k] : -INFINITY;
+                    tM[sp * kMaxGroupHeads + hh] = mk;
+                    tL[sp * kMaxGroupHeads + hh] = live ? l8[k] : 0.0f;
+                    M = fmaxf(M, mk);
+                }
+            }
+        }
+        M = head_max(M);
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        float L = 0.0f;
+        for (int sp = s8; sp < nsp32; sp += 8) {
+            float w = 0.0f;
+            if (sp < P.nsplit) {
+                w = __builtin_amdgcn_exp2f(tM[sp * kMaxGroupHeads + hh] - Mu);
+                L += w * tL[sp * kMaxGroupHeads + hh];
+            }
+            sW[hh * nsp32 + sp] = w;
+        }
+        L = head_sum(L);
+        if (s8 == 0) {
+            sHead[hh] = M;
+            sHead[kMaxGroupHeads + hh] = L;
+        }
+        PROF(13);
+    }
+    __syncthreads();
+    PROF(14);
     for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
         const int hh = idx >> 7, c = idx & 127;
         const int hq = hk * g + hh;
-        const int64_t row0 = bi * P.h + hq;
-        float M = -INFINITY, sum = 0.0f, o = 0.0f;
+        float O = 0.0f;
         for (int s0 = 0; s0 < P.nsplit; s0 += 32) {
-            float v[32], e[32];
-#pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                const int sidx = min(s0 + k, P.nsplit - 1);
-                v[k] = ld_dev(&P.o_part[(sidx * hstride + row0) * kHeadDim + c]);
-                e[k] = ld_dev(&P.lse_part[sidx * hstride + row0]);
+            if (idx != tid || s0 != 0) {
+                load_partials(v0, P.o_part, (row00 + hh) * kHeadDim + c, hstride * kHeadDim, s0, P.nsplit);
             }
-            float mb = -INFINITY;
 #pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                if (s0 + k >= P.nsplit) e[k] = -INFINITY;
-                mb = fmaxf(mb, e[k]);
+            for (int k = 0; k < 32; k += 4) {
+                const f4 w4 = *reinterpret_cast<const f4*>(&sW[hh * nsp32 + s0 + k]);
+                O += w4[0] * v0[k];
+                O += w4[1] * v0[k + 1];
+                O += w4[2] * v0[k + 2];
+                O += w4[3] * v0[k + 3];
             }
-            const float Mn = fmaxf(M, mb);
-            const float Mu = (Mn == -INFINITY) ? 0.0f : Mn;
-            const float a = __expf(M - Mu);
-            sum *= a;
-            o *= a;
-#pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                const float w = __expf(e[k] - Mu);
-                sum += w;
-                o += w * v[k];
-            }
-            M = Mn;
         }
-        const bool none = (sum == 0.0f || sum != sum);
-        P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(none ? 0.0f : o / sum);
-        if (c == 0 && P.lse) P.lse[row0] = none ? INFINITY : __logf(sum) + M;
+        const float M = sHead[hh], L = sHead[kMaxGroupHeads + hh];
+        const bool none = !(L > 0.0f);
+        P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(none ? 0.0f : O / L);
+        if (c == 0 && P.lse) {
+            P.lse[row00 + hh] = none ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+        }
     }
     PROF(7);
     PROF_FLUSH();

@@ -34,8 +34,8 @@ struct FwdParams {
     const int* seqlens;
     const int* reslens;
     int seqlen, reslen;
-    float* o_part;      // [split][b][h][128] normalised partial outputs
-    float* lse_part;    // [split][b][h] natural-log LSE of each split
+    float* o_part;      // [split][b][h][128] partial outputs, relative to the split's own maximum
+    float* ml_part;     // [split][b][h][2] maximum (base-2 units) and sum of each split
     int* tickets;       // [b][h_k] arrival counters, zero between calls
     uint16_t* out;
     int64_t out_sb, out_sh;

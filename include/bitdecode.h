@@ -88,7 +88,7 @@ typedef struct bitdecode_fwd_args {
     int32_t b, h, h_k, d;      /* d must be 128, h % h_k == 0, h / h_k <= 8                 */
     int32_t bits, group_size, dtype;
     float softmax_scale;
-    int32_t num_splits;        /* 0 = choose (bitdecode_num_splits)                         */
+    int32_t num_splits;        /* 0 = choose (bitdecode_num_splits); at most 512            */
 } bitdecode_fwd_args;
 
 int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
