@@ -23,11 +23,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the split-KV kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/fwd_splitkv_llama3-8b-gqa-32k-4bit-g128.md): the counters read 18090.8 and 560.25 per
-# dispatch; a 256 MiB device copy in the same runs reads 131089 and 262144, i.e. the fetch counter
-# is in units of 2 KiB and the write counter in KiB.
+# (profiles/fwd_splitkv_and_qpack_llama3-8b-gqa-32k-4bit-g128.md): the counters read 18092.2 and
+# 592.25 per dispatch; a 256 MiB device copy in the same runs reads 131087 and 262144, i.e. the fetch
+# counter is in units of 2 KiB and the write counter in KiB.
 MEASURED_TRAFFIC_BYTES = {
-    "llama3-8b-gqa-32k-4bit-g128": int(18090.8 * 2048 + 560.25 * 1024),
+    "llama3-8b-gqa-32k-4bit-g128": int(18092.2 * 2048 + 592.25 * 1024),
 }
 
 WORKLOADS = {
@@ -134,6 +134,7 @@ def main():
     ap.add_argument("--no-rotate", action="store_true", help="reuse one KV cache (stays in the 256 MB Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fp16", action="store_true", help="skip the fp16-KV baseline leg")
+    ap.add_argument("--no-qpack", action="store_true", help="skip the quantize-pack kernel leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three plain 256 MiB device copies (a kernel of known traffic, used to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -157,7 +158,7 @@ def main():
     # enough distinct caches that consecutive steps cannot be served from the Infinity Cache
     nbuf = 1 if args.no_rotate else max(2, math.ceil(320e6 / total_bytes))
     nbuf = min(nbuf, 16)
-    plans, keep = [], []
+    plans, keep, srcs = [], [], []
     q0 = k0 = v0 = None
     for i in range(nbuf):
         q, k, v = make_inputs(b, h, h_k, S + R, seed=i, dtype=dtype)
@@ -172,6 +173,8 @@ def main():
                                     k_residual=kres, v_residual=vres, num_splits=args.num_splits)
         plans.append(plan)
         keep.append((cache, kres, vres))
+        if i < 2 and not args.no_qpack:
+            srcs.append((kd, vd))      # fp16 sources of the first two caches, for the quantize-pack leg
         del kd, vd
     torch.cuda.synchronize(dev)
 
@@ -216,6 +219,36 @@ def main():
                      "kernel": "fwd_splitkv_kernel", "algorithmic_bytes": total_bytes,
                      "packed_stream_bytes": packed_bytes, "us_per_step_events": round(us_step_ev, 3)},
     }
+
+    if not args.no_qpack:
+        # the other kernel of the path: quantize-pack of the whole packed prefix (prefill-side bulk pack)
+        # and of one 128-token block per sequence (the append step of a decode loop); every call rewrites
+        # a cache with the bytes it already holds
+        def pack_all(i):
+            j = i % len(srcs)
+            kd, vd = srcs[j]
+            c = keep[j][0]
+            kvcache_pack_int(kd[:, :S], c[0], c[1], vd[:, :S], c[2], c[3], None, None, S, "k-channel", gs, bits)
+
+        def pack_block(i):
+            j = i % len(srcs)
+            kd, vd = srcs[j]
+            c = keep[j][0]
+            kvcache_pack_int(kd[:, S - 128:S], c[0], c[1], vd[:, S - 128:S], c[2], c[3], None, None, 128,
+                             "k-channel", gs, bits, dst_offset=S - 128)
+
+        n_pack = max(10, args.steps // 4)
+        _, ep, _ = time_steps(pack_all, n_pack, 3, not args.no_graph)
+        _, ea, _ = time_steps(pack_block, args.steps, args.warmup, not args.no_graph)
+        us_pack, us_app = ep / n_pack * 1e6, ea / args.steps * 1e6
+        rd = b * h_k * S * 128 * 2 * 2
+        gbs = (rd + packed_bytes) / (us_pack * 1e-6) / 1e9
+        result["qpack"] = {
+            "kernel": "qpack_kernel", "bound": "hbm", "tokens": S, "us_per_call": round(us_pack, 3),
+            "bytes_read": rd, "bytes_written": packed_bytes, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "append_128_tokens_us_per_call": round(us_app, 3)}
+        srcs.clear()
 
     if not args.no_fp16:
         # fp16-KV decode on the same GPU: the library's own fp16 split-KV path over all S+R tokens,

@@ -117,3 +117,24 @@ def test_decode_many_chunks_per_wave(device, bits, gs):
         out = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns)
         err = np.abs(out.float().cpu().numpy() - want).max()
         assert err < ATOL, (ns, err)
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 128), (4, 32), (2, 128), (2, 32)])
+def test_decode_many_splits(device, bits, gs):
+    """More splits than one batch of the final merge handles at once (33, 70), and more splits than
+    packed units (100 over 40 or 80 units: most splits are empty and must contribute nothing).  The
+    result and the LSE must not depend on the split count."""
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, S, R = 2, 8, 2, 128 * 40, 48
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=33)
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, want_lse = O.attend_ref(q, k_hat, v_hat, SCALE, k[:, S:], v[:, S:])
+    kres, vres = H.to_dev(k[:, S:], "fp16", device), H.to_dev(v[:, S:], "fp16", device)
+    for ns in (33, 70, 100, 512):
+        out, lse = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits,
+                                   k_residual=kres, v_residual=vres, num_splits=ns, return_lse=True)
+        err = np.abs(out.float().cpu().numpy() - want).max()
+        assert err < ATOL, (ns, err)
+        np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=2e-3, rtol=1e-4)
