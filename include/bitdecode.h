@@ -35,7 +35,9 @@ enum { BITDECODE_FP16 = 0, BITDECODE_BF16 = 1 };
  * Replaces kvcache_qpack<num_bits> (csrc/bit_decode/decode_api.cpp:517-603) and the kernel it
  * launches (csrc/bit_decode/src/flash_fwd_kernel.h:732-1091).  K is quantized per channel over
  * groups of group_size consecutive tokens, V per token over groups of group_size consecutive
- * channels; scale and zero (= group minimum) are stored in the element type. */
+ * channels; scale and zero (= group minimum) are rounded to the element type and stored as fp16
+ * bit patterns (for bf16: the bf16 value converted to fp16, the same number inside the fp16
+ * normal range). */
 typedef struct bitdecode_qpack_args {
     const void* k;             /* [b, n_tokens, h_k, 128] fp16/bf16, last dim contiguous    */
     const void* v;
