@@ -238,3 +238,19 @@ def test_algorithmic_bytes_match_published_table():
     assert O.algorithmic_bytes(1, 32, 8, 32768, 128, 4, 128) == 36_192_256
     assert O.algorithmic_bytes(1, 32, 8, 131072, 128, 2, 64) == 84_426_752
     assert O.algorithmic_bytes(8, 64, 8, 8 * 65536, 8 * 128, 2, 128) == 306_446_336
+
+
+def test_roundf_equals_floor_of_biased_sum_for_nonnegative_values():
+    """The pack kernel computes roundf(t), t >= 0, as floor(t + 0.49999997f) in fp32.  Checked against
+    round-half-away for every float in [0.25, 16.5] and a sweep of smaller ones."""
+    c = np.nextafter(np.float32(0.5), np.float32(0))
+    assert c == np.float32(0.49999997)
+    lo, hi = np.float32(0.25).view(np.uint32), np.float32(16.5).view(np.uint32)
+    for start in range(int(lo), int(hi) + 1, 1 << 24):
+        t = np.arange(start, min(start + (1 << 24), int(hi) + 1), dtype=np.uint32).view(np.float32)
+        fl = np.floor(t)
+        want = fl + ((t - fl) >= np.float32(0.5))
+        np.testing.assert_array_equal(np.floor((t + c).astype(np.float32)), want)
+        np.testing.assert_array_equal(want, O.roundf(t))
+    small = np.arange(0, int(lo), 4099, dtype=np.uint32).view(np.float32)
+    np.testing.assert_array_equal(np.floor((small + c).astype(np.float32)), np.zeros_like(small))
