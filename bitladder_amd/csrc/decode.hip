@@ -249,20 +249,30 @@ struct UnitCfg {
     static constexpr int TPG = GS / 16;                      // tiles per K group
     static constexpr int NGU = UT > GS ? UT / GS : 1;        // K groups a unit touches
     static constexpr int NCG = kHeadDim / GS;                // V channel groups
-    static constexpr int KPB = NGU * kKParamGroupBytes;      // K parameter bytes per unit
-    static constexpr int VPB = UT * NCG * 4;                 // V parameter bytes per unit
-    static constexpr int PROWS = (KPB + VPB + 1023) / 1024;  // 1 KB rows holding [K params | V params]
-    static constexpr int REGION = 8192 + PROWS * 1024;       // LDS bytes per wave: K codes, V codes, params
+    static constexpr int KPB = unit_k_param_bytes(BITS, GS); // K parameter bytes per unit
+    static constexpr int VPB = unit_v_param_bytes(BITS, GS); // V parameter bytes per unit
+    static constexpr int NKP = (KPB + 1023) / 1024;          // load instructions for the K parameters
+    static constexpr int NVP = (VPB + 1023) / 1024;          // ... for the V parameters
+    static constexpr int KSIDE = NKP + 4;                    // loads of a unit's K side (parameters, 4 code rows)
+    static constexpr int VSIDE = NVP + 4;                    // ... of its V side
+    // LDS region of a wave: K rows | V rows | K parameters, two slots | V parameters
+    static constexpr int OFF_KP = 8192, OFF_VP = 8192 + 2 * KPB;
+    static constexpr int REGION = unit_region_bytes(BITS, GS);
     static constexpr int NW = decode_waves(BITS, GS);        // waves per workgroup
-    static_assert(REGION == unit_region_bytes(BITS, GS), "layout.h and the kernel disagree on the LDS region");
+    static_assert(REGION == OFF_VP + VPB && REGION % 256 == 0, "region layout");
+    static_assert(NW % 4 == 0, "the merge reads four wave weights per LDS access");
 };
 
-// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_base + 16*l.
+// 16 bytes per lane from global memory straight into LDS: lane l reads base + OFFSET + 16*l and its
+// data lands at lds_base + OFFSET + 16*l (the instruction's immediate offset applies to both sides).  The base is wave-uniform and travels in SGPRs, the per-lane part is
+// one shared VGPR (lane16 = 16*lane), so the addresses of a whole unit cost no vector registers.
 // M0 carries the LDS byte address of the row.
-__device__ __forceinline__ void dma_row(const void* gaddr_of_lane, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+template <int OFFSET>
+__device__ __forceinline__ void dma_row(const uint8_t* base, uint32_t lane16, uint32_t lds_base) {
+    static_assert(OFFSET >= 0 && OFFSET < 4096, "immediate offset field");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
                  :
-                 : "v"(gaddr_of_lane), "s"(lds_base)
+                 : "v"(lane16), "s"(base), "s"(lds_base), "n"(OFFSET)
                  : "memory", "m0");
 }
 
@@ -271,6 +281,25 @@ __device__ __forceinline__ void dma_row(const void* gaddr_of_lane, uint32_t lds_
 template <int N>
 __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// the same for a count that is a constant only after loop unrolling (the switch folds away)
+__device__ __forceinline__ void wait_vm_n(int n) {
+    switch (n) {
+        case 0: wait_vm<0>(); break;
+        case 1: wait_vm<1>(); break;
+        case 2: wait_vm<2>(); break;
+        case 3: wait_vm<3>(); break;
+        case 4: wait_vm<4>(); break;
+        case 5: wait_vm<5>(); break;
+        case 6: wait_vm<6>(); break;
+        case 7: wait_vm<7>(); break;
+        case 8: wait_vm<8>(); break;
+        case 9: wait_vm<9>(); break;
+        case 10: wait_vm<10>(); break;
+        case 11: wait_vm<11>(); break;
+        default: wait_vm<0>(); break;      // waiting for more than needed is always safe
+    }
 }
 
 // A 16-byte global load the compiler does not track (so that its automatic waits do not count
@@ -305,11 +334,12 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
         (const __attribute__((address_space(3))) void*)p));
 }
 
-// The loads of unit u, in the order they are consumed: the parameter rows, then per 64-token step
-// its K rows and its V rows.  The first unit of a wave is issued in one go; for later units of a
-// two-step unit the second step is issued while the first is being computed (a wave stalls while
-// the memory pipeline will not take its next load, so it queues what it needs next and keeps the
-// VALU busy in between).
+// The loads of a unit, in the order they are consumed: K side (K parameters, four K code rows), then
+// V side (V parameters, four V code rows).  A wave issues both sides of its first unit at once.
+// After that the next unit's K side is issued as soon as the current unit's last QK^T has read the
+// K rows, into the same rows and into the other K-parameter slot, and its V side as soon as the last
+// PV has read the V rows and V parameters: the next unit is on its way while the current one is
+// being computed, without a second code buffer.
 template <int BITS, int GS>
 struct UnitAddr {
     const uint8_t* kc;
@@ -318,49 +348,45 @@ struct UnitAddr {
     const uint8_t* vp;
 };
 template <int BITS, int GS>
-__device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int64_t bh, int u, int lane) {
+__device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int64_t bh, int u) {
     using C = UnitCfg<BITS, GS>;
     const int ci = u / C::UPC, uic = u % C::UPC;
-    UnitAddr<BITS, GS> A;
-    A.kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096 + lane * 16;
-    A.vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096 + lane * 16;
+    UnitAddr<BITS, GS> A;      // wave-uniform: everything here lives in SGPRs
+    A.kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
+    A.vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
     A.kp = P.k_params + bh * P.kparams_bh +
            (static_cast<int64_t>(ci) * (kChunk / GS) + (uic * C::UT) / GS) * kKParamGroupBytes;
     A.vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS) + uic * C::VPB;
     return A;
 }
-template <int BITS, int GS>
-__device__ __forceinline__ void issue_params(const UnitAddr<BITS, GS>& A, int lane, uint32_t region) {
-    using C = UnitCfg<BITS, GS>;
-#pragma unroll
-    for (int r = 0; r < C::PROWS; ++r) {
-        const int o = r * 1024 + lane * 16;                   // byte offset inside [K params | V params]
-        const uint8_t* src =
-            o < C::KPB ? A.kp + o : (o < C::KPB + C::VPB ? A.vp + (o - C::KPB) : A.kp + (o & (C::KPB - 1)));
-        dma_row(src, region + 8192 + r * 1024);
+// BYTES contiguous bytes (a multiple of 256) into LDS: whole 1 KB rows, the last one with only the
+// lanes that still have data.  Lane 0 always takes part, so every wave executes every instruction
+// and the vmcnt bookkeeping below holds.
+template <int BYTES, int R = 0>
+__device__ __forceinline__ void dma_bytes(const uint8_t* src, uint32_t lane16, uint32_t lds_dst) {
+    if constexpr (R * 1024 < BYTES) {
+        constexpr int left = BYTES - R * 1024;
+        if (left >= 1024 || lane16 < left) dma_row<R * 1024>(src, lane16, lds_dst);
+        dma_bytes<BYTES, R + 1>(src, lane16, lds_dst);
     }
 }
 template <int BITS, int GS>
-__device__ __forceinline__ void issue_step(const UnitAddr<BITS, GS>& A, uint32_t region, int step) {
+__device__ __forceinline__ void issue_kside(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region, int kslot) {
     using C = UnitCfg<BITS, GS>;
-#pragma unroll
-    for (int r = 0; r < C::RPS; ++r) dma_row(A.kc + (step * C::RPS + r) * 1024, region + (step * C::RPS + r) * 1024);
-#pragma unroll
-    for (int r = 0; r < C::RPS; ++r) {
-        dma_row(A.vc + (step * C::RPS + r) * 1024, region + 4096 + (step * C::RPS + r) * 1024);
-    }
+    dma_bytes<C::KPB>(A.kp, lane16, region + C::OFF_KP + kslot * C::KPB);
+    dma_row<0>(A.kc, lane16, region);
+    dma_row<1024>(A.kc, lane16, region);
+    dma_row<2048>(A.kc, lane16, region);
+    dma_row<3072>(A.kc, lane16, region);
 }
-// FULL: params and every step; otherwise params and step 0 (compute_unit issues the rest)
-template <int BITS, int GS, bool FULL>
-__device__ __forceinline__ void issue_unit(const UnitAddr<BITS, GS>& A, int lane, uint32_t region) {
-    issue_params<BITS, GS>(A, lane, region);
-    issue_step<BITS, GS>(A, region, 0);
-    if (FULL && UnitCfg<BITS, GS>::NSTEP > 1) issue_step<BITS, GS>(A, region, 1);
-}
-template <int BITS, int GS, bool FULL>
-constexpr int unit_loads() {
+template <int BITS, int GS>
+__device__ __forceinline__ void issue_vside(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region) {
     using C = UnitCfg<BITS, GS>;
-    return C::PROWS + 2 * C::RPS * (FULL ? C::NSTEP : 1);
+    dma_bytes<C::VPB>(A.vp, lane16, region + C::OFF_VP);
+    dma_row<0>(A.vc, lane16, region + 4096);
+    dma_row<1024>(A.vc, lane16, region + 4096);
+    dma_row<2048>(A.vc, lane16, region + 4096);
+    dma_row<3072>(A.vc, lane16, region + 4096);
 }
 
 // Per-group state of the K side: Q with the group's scale folded in (exact hi/lo split) and the
@@ -414,39 +440,38 @@ __device__ __forceinline__ void start_group(KGroup& G, const uint8_t* kpar, cons
 
 // One packed unit from the wave's LDS region, in 64-token steps: S^T tiles of the step, online
 // softmax update, O^T += V^T P^T for the same tokens.  Scores stay in q.k units; the softmax
-// scale is applied inside the exponent.  FULL: all loads of the unit are already in flight.
-template <int BITS, int GS, bool BF16, bool FULL>
-__device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, const UnitAddr<BITS, GS>& A,
-                                             const QRows& Q, const FwdParams& P, int lane, bool lo_part,
-                                             const Magic& mg, WaveState<kHeadDim / GS>& st,
+// scale is applied inside the exponent.  On entry both sides of the unit are in flight or landed
+// (queue order: K side, V side).  With HAS_NEXT the two sides of the wave's next unit are issued
+// from here (see above); kslot says which K-parameter slot the current unit uses.
+template <int BITS, int GS, bool BF16, bool HAS_NEXT>
+__device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, int kslot,
+                                             const UnitAddr<BITS, GS>& next, const QRows& Q, const FwdParams& P,
+                                             int lane, bool lo_part, const Magic& mg, WaveState<kHeadDim / GS>& st,
                                              unsigned long long* phase_ts = nullptr) {
     using C = UnitCfg<BITS, GS>;
     constexpr int NCG = C::NCG, TPS = C::TPS, NKS = C::NKS, TPG = C::TPG, CTPG = GS / 16;
-    constexpr int NSTEP = C::NSTEP, RPS = C::RPS, STEP_LOADS = 2 * RPS;
+    constexpr int NSTEP = C::NSTEP, RPS = C::RPS;
     const int kg = lane >> 4;
     const h8 noff = -code_offsets<BITS>();
     const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
     const uint32_t hi_cols = lo_part ? 0u : 0xffffffffu;
     const u4* kcode = reinterpret_cast<const u4*>(reg) + lane;             // row r: kcode[64 * r]
     const u4* vcode = reinterpret_cast<const u4*>(reg + 4096) + lane;
-    const uint8_t* kpar = reg + 8192;
-    const uint8_t* vpar = reg + 8192 + C::KPB + kg * 16;
+    const uint8_t* kpar = reg + C::OFF_KP + kslot * C::KPB;
+    const uint8_t* vpar = reg + C::OFF_VP + kg * 16;
 
-    // the parameter rows lead the queue: the first K group is prepared while the code rows arrive
-    wait_vm<STEP_LOADS * (FULL ? NSTEP : 1)>();
+    // the K parameters lead the queue: the first K group is prepared while the code rows arrive
+    wait_vm<4 + C::VSIDE>();
     PHASE(8);
     KGroup G;
     start_group<BITS, BF16>(G, kpar, Q, kg);
     (void)phase_ts;
 #pragma unroll
     for (int step = 0; step < NSTEP; ++step) {
-        // loads allowed in flight when the K rows of this step are needed: its V rows and later steps
-        constexpr int kLaterFull = STEP_LOADS * (NSTEP - 1);
-        if (step == 0) {
-            if (FULL) wait_vm<RPS + kLaterFull>(); else wait_vm<RPS>();
-        } else {
-            wait_vm<RPS>();
-        }
+        constexpr int kLast = NSTEP - 1;
+        // still allowed in flight: the K rows of later steps and the whole V side
+        wait_vm<4 - RPS + C::VSIDE>();
+        if (step > 0) wait_vm<C::VSIDE>();
         PHASE(9 + 3 * step);
         float t[4 * TPS];
 #pragma unroll
@@ -473,7 +498,8 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
 #pragma unroll
             for (int r = 0; r < 4; ++r) t[4 * tt + r] = acc[r] + partner(acc[r]);   // hi + lo
         }
-        if (!FULL && step + 1 < NSTEP) issue_step<BITS, GS>(A, region_lds, step + 1);
+        // every K row and this unit's K parameters have been read: the next unit's K side may land
+        if (HAS_NEXT && step == kLast) issue_kside<BITS, GS>(next, lane * 16, region_lds, kslot ^ 1);
         PHASE(10 + 3 * step);
 
         softmax_step<4 * TPS, NCG>(t, P.scale_log2, st);
@@ -493,7 +519,8 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
             st.l = mfma32(ones, pz[ks], st.l);
         }
         PHASE(11 + 3 * step);
-        if (step + 1 < NSTEP) wait_vm<STEP_LOADS>(); else wait_vm<0>();
+        // still allowed in flight: the V rows of later steps and, once issued, the next unit's K side
+        wait_vm_n((HAS_NEXT && step == kLast) ? C::KSIDE : 4 - (step + 1) * RPS);
 #pragma unroll
         for (int cg = 0; cg < NCG; ++cg) {
             h8 pp[NKS];
@@ -526,6 +553,8 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
             }
         }
     }
+    // every V row and the V parameters have been read: the next unit's V side may land
+    if (HAS_NEXT) issue_vside<BITS, GS>(next, lane * 16, region_lds);
     PHASE(15);
 }
 
@@ -747,9 +776,10 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     }
     UnitAddr<BITS, GS> A;
     if (u < u1) {
-        A = unit_addr<BITS, GS>(P, bh, u, lane);
-        issue_unit<BITS, GS, true>(A, lane, region_lds);
-        wait_then_take<unit_loads<BITS, GS, true>()>(qa, qb, qa_raw, qb_raw);
+        A = unit_addr<BITS, GS>(P, bh, u);
+        issue_kside<BITS, GS>(A, lane * 16, region_lds, 0);
+        issue_vside<BITS, GS>(A, lane * 16, region_lds);
+        wait_then_take<C::KSIDE + C::VSIDE>(qa, qb, qa_raw, qb_raw);
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
     }
@@ -782,19 +812,20 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     if (u < u1) {
         const Magic mg;
 #ifdef BITDECODE_PROF
-        wait_vm<2 * C::RPS * C::NSTEP>();   // parameter rows have arrived
+        wait_vm<4 + C::VSIDE>();   // K parameters have arrived
         PROF(2);
-#endif
-#ifdef BITDECODE_PROF
-        compute_unit<BITS, GS, BF16, true>(region, region_lds, A, Q, P, lane, lo_part, mg, st, prof_ts);
+        unsigned long long* phase_ts = prof_ts;
 #else
-        compute_unit<BITS, GS, BF16, true>(region, region_lds, A, Q, P, lane, lo_part, mg, st);
+        unsigned long long* phase_ts = nullptr;
 #endif
-        for (u += NW; u < u1; u += NW) {
-            A = unit_addr<BITS, GS>(P, bh, u, lane);
-            issue_unit<BITS, GS, false>(A, lane, region_lds);
-            compute_unit<BITS, GS, BF16, false>(region, region_lds, A, Q, P, lane, lo_part, mg, st);
+        int kslot = 0;
+        for (int un = u + NW; un < u1; un += NW) {        // units that have a successor: it is fetched from inside
+            A = unit_addr<BITS, GS>(P, bh, un);
+            compute_unit<BITS, GS, BF16, true>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
+            kslot ^= 1;
+            phase_ts = nullptr;
         }
+        compute_unit<BITS, GS, BF16, false>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
     }
     PROF(3);
     // ---- fp16 window tiles of this wave (the region becomes the V-transpose slab)

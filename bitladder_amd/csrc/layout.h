@@ -57,15 +57,21 @@ constexpr int64_t v_param_region_bytes(int64_t S, int gs) { return S * (kHeadDim
 
 // ---- decode work units (shared by the kernel and the host-side split choice)
 // A decode wave streams units of 4 KB of K codes + 4 KB of V codes + their parameters through its
-// private LDS region: 64 tokens at 4 bits, 128 tokens at 2 bits.
+// private LDS region: 64 tokens at 4 bits, 128 tokens at 2 bits.  The region holds the code rows, two
+// slots of K parameters (the next unit's are fetched while the current ones are in use) and one slot of
+// V parameters.
 constexpr int unit_tokens(int bits) { return bits == 4 ? 64 : 128; }
-constexpr int unit_region_bytes(int bits, int gs) {
+constexpr int unit_k_param_bytes(int bits, int gs) {
     const int ut = unit_tokens(bits);
-    const int kpb = (ut > gs ? ut / gs : 1) * kKParamGroupBytes;
-    const int vpb = ut * (kHeadDim / gs) * 4;
-    return 8192 + (kpb + vpb + 1023) / 1024 * 1024;
+    return (ut > gs ? ut / gs : 1) * kKParamGroupBytes;
+}
+constexpr int unit_v_param_bytes(int bits, int gs) { return unit_tokens(bits) * (kHeadDim / gs) * 4; }
+constexpr int unit_region_bytes(int bits, int gs) {
+    return 8192 + 2 * unit_k_param_bytes(bits, gs) + unit_v_param_bytes(bits, gs);
 }
 // waves per decode workgroup: as many as 160 KB of LDS (less shared scratch) and the register file allow
-constexpr int decode_waves(int bits, int gs) { return unit_region_bytes(bits, gs) <= 9216 ? 16 : 12; }
+constexpr int decode_waves(int bits, int gs) {
+    return unit_region_bytes(bits, gs) <= 9728 ? 16 : (unit_region_bytes(bits, gs) <= 12288 ? 12 : 8);
+}
 
 }  // namespace bitdecode

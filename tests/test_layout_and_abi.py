@@ -207,8 +207,8 @@ def test_split_choice_and_workspace_size():
     assert lib.bitdecode_num_splits(64, 8, 4096, 128, 256, 4, 128) == 1
     # never more splits than there is work for: 4 units of 64 tokens -> one workgroup
     assert lib.bitdecode_num_splits(1, 1, 256, 0, 256, 4, 128) == 1
-    # 48 units over 16 waves -> 3 splits
-    assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256, 4, 128) == 3
+    # 48 units, at least one unit for every second of the 16 waves -> 6 splits
+    assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256, 4, 128) == 6
     assert lib.bitdecode_num_splits(1, 1, 1024, 0, 256, 3, 128) == -1
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 256 + 32 * 32 * 130 * 4
