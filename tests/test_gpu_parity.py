@@ -138,3 +138,53 @@ def test_decode_many_splits(device, bits, gs):
         err = np.abs(out.float().cpu().numpy() - want).max()
         assert err < ATOL, (ns, err)
         np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=2e-3, rtol=1e-4)
+
+
+def test_plan_and_pack_replay_in_hip_graph(device):
+    """A decode plan (split workspace included) and an append-pack call are captured in one HIP graph
+    and replayed several times with eager work and synchronisations in between; every replay must
+    reproduce the eager result bit for bit, also after the inputs behind the captured pointers change."""
+    from bitladder_amd import kvcache_pack_int, plan_fwd_kvcache_int
+    b, h, h_k, S, R, bits, gs = 2, 8, 2, 128 * 12, 128, 4, 128
+    q, k, v = O.make_inputs(b, h, h_k, S + 128, R, seed=44)
+    kd, vd = H.to_dev(k, "fp16", device), H.to_dev(v, "fp16", device)
+    qd = H.to_dev(q, "fp16", device)
+    cache = H.alloc_cache(b, S + 128, h_k, bits, gs, device)
+    kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S, "k-channel", gs, bits)
+    new_k, new_v = kd[:, S:S + 128].clone(), vd[:, S:S + 128].clone()      # block appended inside the graph
+    kres, vres = kd[:, S + 128:].contiguous(), vd[:, S + 128:].contiguous()
+    plan = plan_fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, seqlen_k=S + 128,
+                                k_residual=kres, v_residual=vres, num_splits=5)
+
+    def step():
+        kvcache_pack_int(new_k, cache[0], cache[1], new_v, cache[2], cache[3], None, None, 128, "k-channel", gs,
+                         bits, dst_offset=S)
+        return plan.run()
+
+    eager = step().clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream(device).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step()
+    for rep in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        # eager work between replays, then new contents behind the captured pointers
+        _ = (kd.float().sum() + vd.float().sum()).item()
+        if rep == 1:
+            qd.mul_(-0.5)
+            new_k.copy_(kd[:, 128:256])
+            new_v.copy_(vd[:, 128:256])
+            eager = step().clone()
+            torch.cuda.synchronize()
+    want_cache = H.alloc_cache(b, S + 128, h_k, bits, gs, device)
+    kvcache_pack_int(torch.cat([kd[:, :S], new_k], 1), want_cache[0], want_cache[1], torch.cat([vd[:, :S], new_v], 1),
+                     want_cache[2], want_cache[3], None, None, S + 128, "k-channel", gs, bits)
+    for a, c in zip(cache, want_cache):
+        assert torch.equal(a, c)
