@@ -5,11 +5,12 @@
 //
 //  * A workgroup owns one (split, kv-head, batch).  Each wave streams whole work units of that
 //    split: 64 packed tokens at 4 bits / 128 at 2 bits (about 9 KB with their parameters), or
-//    16-token tiles of the fp16 window.  A unit is fetched with nine direct-to-LDS loads
+//    16-token tiles of the fp16 window.  A unit is fetched with ten direct-to-LDS loads
 //    (global_load_lds_dwordx4: 64 lanes x 16 B = one contiguous 1 KB row each, no staging
 //    registers) into the wave's private LDS region and read back 16 bytes per lane just before
-//    it is unpacked.  With no load-staging registers the kernel fits 3-4 waves per SIMD, which is
-//    what hides the load latency: a wave that waits for its unit leaves the VALU to the others.
+//    it is unpacked; the next unit of the wave is requested from inside the current one, as soon
+//    as the rows it will overwrite have been read.  With no load-staging registers the kernel
+//    fits 3-4 waves per SIMD: a wave that waits for its unit leaves the VALU to the others.
 //  * Both products are computed transposed on v_mfma_f32_16x16x32_f16:
 //        S^T = K * Q^T   (A = K codes, row = token; B = Q, column = query head of the GQA group)
 //        O^T = V^T * P^T (A = V codes, row = channel; B = P^T)
@@ -29,11 +30,12 @@
 //  * The offset/zero biases and the softmax row sums are themselves computed on the MFMA pipe
 //    (A operand = the zero vector / the constant offsets / ones), which keeps the VALU for the
 //    code unpacking; this kernel is VALU-issue bound long before it is MFMA bound.
-//  * Online softmax in base 2 per head (softmax.h:250-310) in steps of 32 tokens (64 at 2 bits):
-//    running max shared by the four lanes of a head through two lane-half swaps, accumulators
-//    rescaled only when some head's max actually moved.
-//  * The waves of a workgroup merge through LDS; splits merge in the same launch: the workgroup
-//    that draws the last ticket of a (batch, kv-head) combines all partials.
+//  * Online softmax in base 2 per head (softmax.h:250-310) in steps of 64 tokens: running max
+//    shared by the four lanes of a head through two lane-half swaps, accumulators rescaled only
+//    when some head's max actually moved.
+//  * The waves of a workgroup merge through LDS; splits merge in the same launch: every
+//    workgroup publishes its unnormalised (O, max, sum) and the one that draws the last ticket
+//    of a (batch, kv-head) combines all of them.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -107,22 +109,7 @@ __device__ __forceinline__ h8 cvt_h8(u4 raw) {
     }
 }
 
-template <bool BF16>
-__device__ __forceinline__ h8 ld_h8(const void* p) {
-    return cvt_h8<BF16>(*reinterpret_cast<const u4*>(p));
-}
-
 __device__ __forceinline__ u4 ld_u4(const void* p) { return *reinterpret_cast<const u4*>(p); }
-
-__device__ __forceinline__ float dot8(h8 a, h8 b, float c) {
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-        h2 a2 = {a[2 * x], a[2 * x + 1]};
-        h2 b2 = {b[2 * x], b[2 * x + 1]};
-        c = __builtin_amdgcn_fdot2(a2, b2, c, false);
-    }
-    return c;
-}
 
 // The exponent patterns that turn a masked code field into offset + code (fp16).  They are kept
 // in VGPRs behind an empty asm so that (w & mask) | magic becomes one v_and_or_b32 (mask from an
@@ -180,13 +167,6 @@ __device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
 __device__ __forceinline__ float partner(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
 }
-// exact product a*b as hi + lo in fp16; returns the part this column carries
-__device__ __forceinline__ h8 split_mul(h8 a, h8 b, bool lo_part) {
-    const h8 hi = a * b;
-    const h8 lo = __builtin_elementwise_fma(a, b, -hi);
-    return lo_part ? lo : hi;
-}
-
 // max over the four lanes that share a column (lane, lane^16, lane^32, lane^48).
 // v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of
 // its second one, v_permlane32_swap does the same with 32-lane halves; fed two copies of x they
@@ -697,13 +677,15 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 // split-KV kernel: 1-D grid of num_splits * h_k * b workgroups of UnitCfg::NW waves.
 // Split s of a (batch, kv-head) owns packed units [s*ups, (s+1)*ups) dealt round-robin to its
 // waves; the 16-token tiles of the fp16 window are dealt round-robin over ALL waves of the head.
-// With more than one split each workgroup writes a normalised partial and takes a ticket; the
-// workgroup that draws the last ticket of its (batch, kv-head) merges all partials
+// With more than one split each workgroup writes its unnormalised (O, max, sum) and takes a ticket;
+// the workgroup that draws the last ticket of its (batch, kv-head) merges all partials
 // (flash_fwd_kernel.h:1217-1298 formula) and resets the ticket.
 //
-// Dynamic LDS: [NW wave regions of UnitCfg::REGION bytes][q: 8 head rows + a zero row, 256 B each][sM, sL: NW x 8 floats]
-// A wave's region is reused as its V-transpose slab for fp16 tiles and as its slot of the
-// cross-wave merge buffer (g x 128 floats <= 4 KB).
+// Dynamic LDS: [NW wave regions of UnitCfg::REGION bytes][q: 8 head rows + a zero row, 272 B apart]
+// [sM, sL: per-wave max and sum, NW x 8 floats each][sA: merge weights, 8 x NW][sHead: merged max and
+// sum, 2 x 8][last-ticket flag].  A wave's region is reused as its V-transpose slab for fp16 tiles
+// and as its slot of the cross-wave merge buffer (g x 128 floats <= 4 KB); the merging workgroup
+// reuses the regions for the per-split maxima, sums and weights.
 // ---------------------------------------------------------------------------------------------
 template <int BITS, int GS>
 constexpr int fwd_lds_bytes() {
