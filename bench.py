@@ -23,11 +23,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the split-KV kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/fwd_splitkv_and_qpack_llama3-8b-gqa-32k-4bit-g128.md): the counters read 18092.2 and
-# 592.25 per dispatch; a 256 MiB device copy in the same runs reads 131087 and 262144, i.e. the fetch
+# (profiles/fwd_splitkv_and_qpack_llama3-8b-gqa-32k-4bit-g128.md): the counters read 18089.2 and
+# 592.25 per dispatch; a 256 MiB device copy in the same runs reads 131085 and 262144, i.e. the fetch
 # counter is in units of 2 KiB and the write counter in KiB.
 MEASURED_TRAFFIC_BYTES = {
-    "llama3-8b-gqa-32k-4bit-g128": int(18092.2 * 2048 + 592.25 * 1024),
+    "llama3-8b-gqa-32k-4bit-g128": int(18089.2 * 2048 + 592.25 * 1024),
 }
 
 WORKLOADS = {
