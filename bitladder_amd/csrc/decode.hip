@@ -627,14 +627,17 @@ __device__ __forceinline__ float ld_dev(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// partial outputs of splits s0 .. s0+31 (clamped to the last split) for one (head, channel)
-__device__ __forceinline__ void load_partials(float (&v)[32], const float* o_part, int64_t item, int64_t split_stride,
+// partial outputs of splits s0 .. s0+31 (clamped to the last split) for one (head, channel).  The
+// split's base address is wave-uniform (SGPRs) and `item` a 32-bit per-thread offset, so the 32
+// loads need no per-load address arithmetic.
+__device__ __forceinline__ void load_partials(float (&v)[32], const float* o_part, uint32_t item, int64_t split_stride,
                                               int s0, int nsplit) {
-    const float* p = o_part + s0 * split_stride + item;
+    const float* base = o_part + static_cast<int64_t>(s0) * split_stride;
+    const int cnt = min(32, nsplit - s0);
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
-        v[k] = ld_dev(p);
-        if (s0 + k + 1 < nsplit) p += split_stride;
+        v[k] = ld_dev(base + item);
+        if (k + 1 < cnt) base += split_stride;
     }
 }
 // (maximum, sum) pairs of splits s0 + s8 + 8k, k = 0..7 (clamped to the last split), for one head
@@ -947,7 +950,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     const int wl_hh = lane & 7, wl_s8 = lane >> 3;
     const int64_t wl_row = row00 + (wl_hh < g ? wl_hh : 0);
     if (wave == 0) load_ml(m8, l8, P.ml_part, wl_row, hstride, 0, wl_s8, P.nsplit);     // ahead of the bulk loads
-    if (tid < g * kHeadDim) load_partials(v0, P.o_part, (row00 + (tid >> 7)) * kHeadDim + (tid & 127),
+    if (tid < g * kHeadDim) load_partials(v0, P.o_part, static_cast<uint32_t>((row00 + (tid >> 7)) * kHeadDim + (tid & 127)),
                                           hstride * kHeadDim, 0, P.nsplit);
     PROF(12);
     if (wave == 0) {
@@ -993,7 +996,8 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         float O = 0.0f;
         for (int s0 = 0; s0 < P.nsplit; s0 += 32) {
             if (idx != tid || s0 != 0) {
-                load_partials(v0, P.o_part, (row00 + hh) * kHeadDim + c, hstride * kHeadDim, s0, P.nsplit);
+                load_partials(v0, P.o_part, static_cast<uint32_t>((row00 + hh) * kHeadDim + c), hstride * kHeadDim, s0,
+                              P.nsplit);
             }
 #pragma unroll
             for (int k = 0; k < 32; k += 4) {
