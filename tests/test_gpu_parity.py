@@ -188,3 +188,48 @@ def test_plan_and_pack_replay_in_hip_graph(device):
                      want_cache[2], want_cache[3], None, None, S + 128, "k-channel", gs, bits)
     for a, c in zip(cache, want_cache):
         assert torch.equal(a, c)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_decode_random_shapes(device, seed):
+    """Seeded sweep over the argument space: batch, GQA ratio, bits, group size, element type, packed
+    length per sequence (ragged, including empty), window length per sequence, split count and the
+    sign of the softmax scale, each against dequantize-then-attend on the same inputs."""
+    from bitladder_amd import fwd_kvcache_int
+    rng = np.random.default_rng(1000 + seed)
+    bits = int(rng.choice([2, 4]))
+    gs = int(rng.choice([32, 64, 128]))
+    dtype = "bf16" if seed % 3 == 2 else "fp16"
+    h_k = int(rng.choice([1, 2, 3]))
+    g = int(rng.choice([1, 2, 4, 5, 8]))
+    b = int(rng.integers(1, 4))
+    S = 128 * int(rng.integers(1, 20))
+    R = int(rng.choice([0, 16, 77, 128]))
+    ns = int(rng.choice([0, 1, 2, 3, 7, 19]))
+    scale = SCALE * (-1.0 if seed % 4 == 3 else 1.0)
+    h = h_k * g
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=2000 + seed, dtype=dtype)
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs, dtype)
+    cache = _pack_gpu(k, v, bits, gs, dtype, device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    seqlens = (128 * rng.integers(0, S // 128 + 1, b)).astype(np.int32)
+    seqlens[rng.integers(0, b)] = S                       # at least one full-length sequence
+    reslens = rng.integers(0, R + 1, b).astype(np.int32) if R else np.zeros(b, np.int32)
+    if R and seqlens.min() == 0:
+        reslens[seqlens == 0] = np.maximum(reslens[seqlens == 0], 1)     # keep every row non-empty here
+    kres = vres = None
+    kw = dict(seqlens_k=torch.from_numpy(seqlens).to(device), max_seqlen_k=S, num_splits=ns, return_lse=True)
+    if R:
+        kw.update(k_residual=H.to_dev(k[:, S:], dtype, device), v_residual=H.to_dev(v[:, S:], dtype, device),
+                  residual_len=torch.from_numpy(reslens).to(device), max_residual_len=R)
+        kres, vres = k[:, S:], v[:, S:]
+    elif seqlens.min() == 0:
+        seqlens[seqlens == 0] = 128
+        kw["seqlens_k"] = torch.from_numpy(seqlens).to(device)
+    want, want_lse = O.attend_ref(q, k_hat, v_hat, scale, kres, vres, seqlens_k=seqlens,
+                                  res_lens=reslens if R else None)
+    out, lse = fwd_kvcache_int(H.to_dev(q, dtype, device), *cache, None, scale, "k-channel", gs, bits, **kw)
+    tol = ATOL if dtype == "fp16" else 8e-3              # a bf16 output keeps 8 significant bits
+    err = np.abs(out.float().cpu().numpy() - want).max()
+    assert err < tol, (bits, gs, dtype, b, h, h_k, S, R, ns, err)
+    np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=3e-3, rtol=1e-4)
