@@ -14,10 +14,12 @@ ARCH = "gfx950"
 COMMON = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
           # packed-FP32 VALU forms are kept out of the generated code on purpose
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-# the quantizer must be IEEE fp32: no contraction, correctly rounded division
+# the quantizer must be IEEE fp32: no contraction, correctly rounded division;
+# the decode kernel is scheduled for instruction-level parallelism rather than for occupancy (its
+# occupancy is fixed by LDS): 2-3 % faster on the long-context workloads, same register counts
 PER_FILE = {
     "qpack.hip": ["-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"],
-    "decode.hip": [],
+    "decode.hip": ["-mllvm", "-amdgpu-sched-strategy=gcn-max-ilp"],
     "api.hip": [],
 }
 
