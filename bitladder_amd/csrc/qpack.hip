@@ -68,12 +68,13 @@ __device__ __forceinline__ void group_params(float mn, float mx, float M, float&
 // t is never negative here (min is the minimum of the group x belongs to, scale_inv >= 0), and for
 // t >= 0  roundf(t) == floor(t + 0.49999997f)  in fp32 round-to-nearest-even arithmetic: the constant
 // is the float just below 0.5, so t = 0.49999997 stays at 0 while every t = k + 0.5 still reaches
-// k + 1 (checked over every float in [0, 64]).  v_cvt_u32_f32 truncates, saturates and maps NaN to 0,
-// which leaves only the upper clamp.
-__device__ __forceinline__ uint32_t quant_code(float x, float mn, float sinv, uint32_t M) {
+// k + 1 (checked over every float in [0, 64]).  The upper clamp can never act: with d = fl(x - min)
+// <= range = fl(max - min) and scale_inv = fl(M / range), t = fl(d * scale_inv) <= M * (1 + 2^-22),
+// far below M + 0.5; an infinite range gives scale_inv = 0 and t = 0 or NaN, and v_cvt_u32_f32 maps
+// NaN to 0.  The conversion truncates, which is the floor of a non-negative value.
+__device__ __forceinline__ uint32_t quant_code(float x, float mn, float sinv) {
     const float t = __fmul_rn(__fsub_rn(x, mn), sinv);
-    const uint32_t c = static_cast<uint32_t>(__fadd_rn(t, 0.49999997f));
-    return c < M ? c : M;
+    return static_cast<uint32_t>(__fadd_rn(t, 0.49999997f));
 }
 
 template <int BITS, int GS, bool BF16>
@@ -81,7 +82,6 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
     constexpr int NG = kChunk / GS;       // K groups per chunk
     constexpr int NCG = kHeadDim / GS;    // V channel groups per token
     constexpr float M = static_cast<float>((1 << BITS) - 1);
-    constexpr uint32_t MI = (1u << BITS) - 1;
 
     __shared__ __attribute__((aligned(16))) uint16_t tile[kChunk * kRowHalves];
     __shared__ float k_qmin[4][kHeadDim], k_qmax[4][kHeadDim];      // per 32-token quarter
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         float x = to_f32<BF16>(tile[n * kRowHalves + ch0 + i]);
-                        uint32_t code = quant_code(x, k_mn[grp][ch0 + i], k_sinv[grp][ch0 + i], MI);
+                        uint32_t code = quant_code(x, k_mn[grp][ch0 + i], k_sinv[grp][ch0 + i]);
                         const int p = i / 2 + 4 * (i % 2);
                         w |= code << (4 * p);
                     }
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
                         const int j = 2 * jj + e / 8, i = e % 8;
                         const int ch = 32 * j + 8 * kg + i;
                         float x = to_f32<BF16>(tile[n * kRowHalves + ch]);
-                        uint32_t code = quant_code(x, k_mn[grp][ch], k_sinv[grp][ch], MI);
+                        uint32_t code = quant_code(x, k_mn[grp][ch], k_sinv[grp][ch]);
                         const int f = e / 2 + 8 * (e % 2);
                         w |= code << (2 * f);
                     }
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
                     for (int i = 0; i < 8; ++i) {
                         const int tok = 32 * sb + 16 * (i / 4) + 4 * kg + (i % 4);
                         float xv = to_f32<BF16>(tile[tok * kRowHalves + ch]);
-                        uint32_t code = quant_code(xv, v_mn[tok][cg], v_sinv[tok][cg], MI);
+                        uint32_t code = quant_code(xv, v_mn[tok][cg], v_sinv[tok][cg]);
                         const int p = i / 2 + 4 * (i % 2);
                         w |= code << (4 * p);
                     }
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
                     const int ks = e / 8, i = e % 8;
                     const int tok = 64 * sb2 + 32 * ks + 16 * (i / 4) + 4 * kg + (i % 4);
                     float xv = to_f32<BF16>(tile[tok * kRowHalves + ch]);
-                    uint32_t code = quant_code(xv, v_mn[tok][cg], v_sinv[tok][cg], MI);
+                    uint32_t code = quant_code(xv, v_mn[tok][cg], v_sinv[tok][cg]);
                     const int f = e / 2 + 8 * (e % 2);
                     w |= code << (2 * f);
                 }

@@ -54,6 +54,8 @@ static void quant_group(const float* x, long st, int n, int bits, int bf16,
     const float M = (float)((1 << bits) - 1);
     float mx = x[0], mn = x[0];
     for (int i = 1; i < n; ++i) { float t = x[i * st]; mx = fmaxf(mx, t); mn = fminf(mn, t); }
+    /* a zero minimum is -0 if the group holds a -0 (IEEE 754-2019 minimum); libm's fminf may return either */
+    if (mn == 0.0f) { for (int i = 0; i < n; ++i) if (x[i * st] == 0.0f && signbit(x[i * st])) mn = -0.0f; }
     volatile float range = mx - mn;
     volatile float scale_inv = (range > 0.0f) ? (M / range) : 0.0f;
     volatile float sc = (scale_inv == 0.0f) ? 0.0f : 1.0f / scale_inv;

@@ -17,7 +17,9 @@ quantize_group / quantize_kv_ref : pinned (closed forms, invariants, brute-force
     rounding cases, C cross-check).  The reference binary is built with
     --use_fast_math (setup.py:149); the contract here is the IEEE-754 fp32 reading
     of csrc/bit_decode/src/include/qpack.h:224-252, so the exact bits of the CUDA
-    binary's `scale` on rare groups are "parity unpinned".
+    binary's `scale` on rare groups are "parity unpinned".  So is the sign of a
+    stored zero-point that is a zero of a group holding both -0 and +0: the reference
+    reduces with `x < y ? x : y`, order-dependent; here -0 orders below +0.
 dequantize_ref  : pinned (exact small-integer arithmetic).
 attend_ref      : pinned (reduces to softmax(QK^T)V; block-order invariance).
 lse_combine_ref : pinned (closed form, split-count invariance).
@@ -91,6 +93,11 @@ def quantize_group(x: np.ndarray, bits: int, axis: int, dtype: str = "fp16"):
     M = F32((1 << bits) - 1)
     mx = np.max(x, axis=axis, keepdims=True)
     mn = np.min(x, axis=axis, keepdims=True)
+    # signed zeros: the minimum orders -0 below +0 (IEEE 754-2019 minimum).  The reference reduces with
+    # `x < y ? x : y` (qpack.h:11-105), which leaves the sign of a zero minimum to the reduction order;
+    # the value, the scale and every code are the same either way.
+    has_neg_zero = np.any((x == 0) & np.signbit(x), axis=axis, keepdims=True)
+    mn = np.where((mn == 0) & has_neg_zero, F32(-0.0), mn).astype(F32)
     rng = (mx - mn).astype(F32)
     with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
         scale_inv = np.where(rng > 0, M / np.where(rng > 0, rng, F32(1)), F32(0)).astype(F32)

@@ -32,6 +32,9 @@ def _quant(x: torch.Tensor, dim: int, bits: int, dtype: torch.dtype):
     M = float((1 << bits) - 1)
     mx = x.amax(dim=dim, keepdim=True)
     mn = x.amin(dim=dim, keepdim=True)
+    # a zero minimum takes the sign of -0 if the group holds one (IEEE 754-2019 minimum)
+    neg0 = ((x == 0) & torch.signbit(x)).any(dim=dim, keepdim=True)
+    mn = torch.where((mn == 0) & neg0, torch.full_like(mn, -0.0), mn)
     rng = mx - mn
     pos = rng > 0
     # tensor / tensor: torch evaluates `python_scalar / tensor` as reciprocal-then-multiply (two

@@ -233,3 +233,30 @@ def test_decode_random_shapes(device, seed):
     err = np.abs(out.float().cpu().numpy() - want).max()
     assert err < tol, (bits, gs, dtype, b, h, h_k, S, R, ns, err)
     np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=3e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_qpack_ranges_from_subnormal_to_max(device, bits, dtype):
+    """Groups whose range spans 2^-24 .. 2^16 (fp16 subnormals up to +-65504), every group containing its
+    exact minimum and maximum: the codes of the extremes must be 0 and 2^bits - 1, nothing may spill into
+    a neighbouring field, and all bytes must equal the oracle's (which clamps explicitly)."""
+    rng = np.random.default_rng(77 + bits)
+    b, h_k, S, gs = 1, 2, 512, 32
+    e = rng.uniform(-24, 15.9, size=(b, S // gs, 1, h_k, 128))
+    lo = rng.uniform(-1, 1, size=e.shape) * 2.0 ** e
+    u = rng.uniform(0, 1, size=(b, S // gs, gs, h_k, 128))
+    u[:, :, 0], u[:, :, 1] = 0.0, 1.0                                   # exact extremes in every K group
+    k = (lo + u * 2.0 ** e).reshape(b, S, h_k, 128)
+    ev = rng.uniform(-24, 15.9, size=(b, S, h_k, 128 // gs, 1))
+    lov = rng.uniform(-1, 1, size=ev.shape) * 2.0 ** ev
+    uv = rng.uniform(0, 1, size=(b, S, h_k, 128 // gs, gs))
+    uv[..., 0], uv[..., 1] = 0.0, 1.0
+    v = (lov + uv * 2.0 ** ev).reshape(b, S, h_k, 128)
+    k, v = np.clip(k, -65504, 65504).astype(np.float32), np.clip(v, -65504, 65504).astype(np.float32)
+    k, v = O.round_to_storage(k, dtype), O.round_to_storage(v, dtype)
+    want = O.quantize_kv_ref(k, v, bits, gs, dtype)
+    assert want.k_codes.max() == (1 << bits) - 1 and want.v_codes.max() == (1 << bits) - 1
+    cache = _pack_gpu(k, v, bits, gs, dtype, device, S)
+    torch.cuda.synchronize()
+    H.assert_cache_equals_oracle(H.cache_to_numpy(*cache), want)

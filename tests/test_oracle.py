@@ -254,3 +254,22 @@ def test_roundf_equals_floor_of_biased_sum_for_nonnegative_values():
         np.testing.assert_array_equal(want, O.roundf(t))
     small = np.arange(0, int(lo), 4099, dtype=np.uint32).view(np.float32)
     np.testing.assert_array_equal(np.floor((small + c).astype(np.float32)), np.zeros_like(small))
+
+
+def test_zero_minimum_takes_the_sign_of_a_negative_zero():
+    """A group whose minimum is zero and that holds a -0 stores zero = -0 whatever the order of its
+    elements (numpy and C restatements agree); value, scale and codes do not depend on the sign."""
+    x = np.array([[0.0, 1.0, -0.0, 3.0], [-0.0, 1.0, 0.0, 3.0], [0.0, 1.0, 0.0, 3.0]], np.float32)
+    codes, scale, zero = O.quantize_group(x, 4, axis=1)
+    assert np.signbit(zero[:, 0]).tolist() == [True, True, False]
+    np.testing.assert_array_equal(codes, np.tile(np.array([0, 5, 0, 15], np.uint8), (3, 1)))
+    k = np.zeros((1, 128, 1, 128), np.float32)
+    k[0, :, 0, :] = np.linspace(0, 2, 128, dtype=np.float32)[:, None]
+    k[0, 5, 0, 3] = -0.0
+    k[0, 0, 0, 3] = 0.0
+    k = O.round_to_storage(k, "fp16")
+    a = O.quantize_kv_ref(k, k, 4, 128)
+    c = C.quantize_kv_c(k, k, 4, 128, "fp16")
+    assert np.signbit(a.k_zero[0, 0, 0, 3]) and not np.signbit(a.k_zero[0, 0, 0, 4])
+    np.testing.assert_array_equal(np.signbit(a.k_zero), np.signbit(c.k_zero))
+    np.testing.assert_array_equal(np.signbit(a.v_zero), np.signbit(c.v_zero))
