@@ -1022,12 +1022,16 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
 template <int BITS, int GS, bool BF16>
 hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
     constexpr int kLds = fwd_lds_bytes<BITS, GS>();
-    static bool configured = false;      // raising the dynamic-LDS limit is idempotent
-    if (!configured) {
+    // the dynamic-LDS limit is raised once per kernel and device (idempotent, so a race between
+    // two host threads only repeats the call)
+    static bool configured[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || !configured[dev]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return e;
-        configured = true;
+        if (dev >= 0 && dev < 64) configured[dev] = true;
     }
     hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16>), dim3(P.nsplit * P.hk * P.b),
                        dim3(UnitCfg<BITS, GS>::NW * 64), kLds, stream, P);
