@@ -10,3 +10,4 @@ from .interface import (  # noqa: F401
     kvcache_pack_int,
     plan_fwd_kvcache_int,
 )
+from .cache import BitKVCache  # noqa: F401,E402

@@ -90,7 +90,9 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
 
     const int tid = threadIdx.x;
     const int ci_src = blockIdx.x, hk = blockIdx.y, bi = blockIdx.z;
-    const int dst_tok = (P.dst_offsets ? P.dst_offsets[bi] : P.dst_offset) + ci_src * kChunk;
+    const int dst_base = P.dst_offsets ? P.dst_offsets[bi] : P.dst_offset;
+    if (dst_base < 0) return;       // a negative per-sequence offset skips that sequence (whole workgroup)
+    const int dst_tok = dst_base + ci_src * kChunk;
     const int ci = dst_tok / kChunk;
     const int64_t bh = static_cast<int64_t>(bi) * P.hk + hk;
 

@@ -50,7 +50,8 @@ typedef struct bitdecode_qpack_args {
     int32_t b, n_tokens, h_k, d;   /* d must be 128; n_tokens a multiple of 128            */
     int32_t cache_tokens;      /* capacity S of the packed tensors, multiple of 128         */
     int32_t dst_offset;        /* token offset of the first written chunk (multiple of 128) */
-    const int32_t* dst_offsets;/* optional device int32[b]: per-sequence dst offset         */
+    const int32_t* dst_offsets;/* optional device int32[b]: per-sequence dst offset; a
+                                  negative entry skips that sequence                        */
     int32_t bits;              /* 2 or 4                                                    */
     int32_t group_size;        /* 32, 64 or 128                                             */
     int32_t dtype;             /* BITDECODE_FP16 / BITDECODE_BF16                           */
