@@ -233,7 +233,7 @@ def test_num_splits_heuristic_known_answers():
 
 
 def test_algorithmic_bytes_match_published_table():
-    # BASELINE figures: C1 19 939 328, C2 36 192 256, C3 84 426 752, C5 306 446 336
+    # published figures for the four fixed-shape benchmark configurations: 19 939 328, 36 192 256, 84 426 752, 306 446 336
     assert O.algorithmic_bytes(1, 32, 32, 4096, 128, 4, 128) == 19_939_328
     assert O.algorithmic_bytes(1, 32, 8, 32768, 128, 4, 128) == 36_192_256
     assert O.algorithmic_bytes(1, 32, 8, 131072, 128, 2, 64) == 84_426_752
