@@ -67,8 +67,8 @@ def alloc_cache(b, S, h_k, bits, gs, dev):
             torch.zeros((b, 128 // gs, h_k, S), dtype=torch.float32, device=dev))
 
 
-def time_steps(run_step, steps, warmup, use_graph):
-    """Returns (wall seconds, event seconds) for exactly `steps` steps."""
+def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0):
+    """Returns (wall seconds, event seconds, graphed) for exactly `steps` steps."""
     dev = torch.device("cuda:0")
     for i in range(warmup):
         run_step(i)
@@ -102,6 +102,19 @@ def time_steps(run_step, steps, warmup, use_graph):
     e1.record()
     torch.cuda.synchronize(dev)
     t1 = time.perf_counter()
+    if quantile_reps and graph is not None:
+        # spread of the per-step time over further replays of the same graph (outside the timed region)
+        per_step = []
+        for _ in range(quantile_reps):
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b_.record()
+            torch.cuda.synchronize(dev)
+            per_step.append(a.elapsed_time(b_) * 1e3 / steps)
+        per_step.sort()
+        pick = lambda f: round(per_step[min(len(per_step) - 1, int(f * len(per_step)))], 3)
+        time_steps.last_quantiles = {"p20": pick(0.2), "p50": pick(0.5), "p80": pick(0.8), "replays": quantile_reps}
     return t1 - t0, e0.elapsed_time(e1) * 1e-3, graph is not None
 
 
@@ -189,7 +202,7 @@ def main():
         torch.cuda.synchronize(dev)
         del src, dst
 
-    wall, evs, graphed = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    wall, evs, graphed = time_steps(step, args.steps, args.warmup, not args.no_graph, quantile_reps=15)
     us_step = wall / args.steps * 1e6
     us_step_ev = evs / args.steps * 1e6
     achieved = total_bytes / (us_step_ev * 1e-6) / 1e9
@@ -219,6 +232,8 @@ def main():
                      "kernel": "fwd_splitkv_kernel", "algorithmic_bytes": total_bytes,
                      "packed_stream_bytes": packed_bytes, "us_per_step_events": round(us_step_ev, 3)},
     }
+    if getattr(time_steps, "last_quantiles", None):
+        result["us_per_step_quantiles"] = time_steps.last_quantiles
 
     if not args.no_qpack:
         # the other kernel of the path: quantize-pack of the whole packed prefix (prefill-side bulk pack)
