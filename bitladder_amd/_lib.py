@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbitdecode.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 FP16, BF16 = 0, 1
 
 _i32, _i64, _vp, _f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
@@ -26,6 +26,8 @@ class QpackArgs(ctypes.Structure):
         ("cache_tokens", _i32), ("dst_offset", _i32),
         ("dst_offsets", _vp),
         ("bits", _i32), ("group_size", _i32), ("dtype", _i32),
+        ("block_table", _vp), ("block_table_stride", _i64),
+        ("max_pages_per_seq", _i32), ("num_pages", _i32),
     ]
 
 
@@ -48,6 +50,8 @@ class FwdArgs(ctypes.Structure):
         ("bits", _i32), ("group_size", _i32), ("dtype", _i32),
         ("softmax_scale", _f32),
         ("num_splits", _i32),
+        ("block_table", _vp), ("block_table_stride", _i64),
+        ("max_pages_per_seq", _i32), ("num_pages", _i32),
     ]
 
 

@@ -88,6 +88,19 @@ size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 2) * sizeof(float);
 }
 
+// paged cache: cache_tokens is the page size; the table must cover `tokens` per sequence
+static int check_paging(const int32_t* block_table, int64_t stride, int32_t max_pages, int32_t num_pages,
+                        int32_t page_tokens, int32_t tokens) {
+    if (!block_table) return BITDECODE_OK;
+    if (max_pages <= 0 || num_pages <= 0 || stride < max_pages)
+        return fail(BITDECODE_EINVAL, "block_table: %d pages per sequence, stride %lld, pool of %d pages", max_pages,
+                    static_cast<long long>(stride), num_pages);
+    if (static_cast<int64_t>(tokens) > static_cast<int64_t>(max_pages) * page_tokens)
+        return fail(BITDECODE_EINVAL, "block_table covers %d x %d tokens per sequence, %d needed", max_pages, page_tokens,
+                    tokens);
+    return BITDECODE_OK;
+}
+
 int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
@@ -96,15 +109,22 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     if (a->n_tokens % kChunk) return fail(BITDECODE_EINVAL, "n_tokens %d is not a multiple of 128", a->n_tokens);
     if (a->cache_tokens % kChunk || a->cache_tokens <= 0)
         return fail(BITDECODE_EINVAL, "cache_tokens %d is not a positive multiple of 128", a->cache_tokens);
+    // tokens one sequence can hold: the tensor capacity, or what its row of the block table covers
+    const int64_t capacity = a->block_table ? static_cast<int64_t>(a->max_pages_per_seq) * a->cache_tokens
+                                            : a->cache_tokens;
     if (!a->dst_offsets) {
         if (a->dst_offset < 0 || a->dst_offset % kChunk)
             return fail(BITDECODE_EINVAL, "dst_offset %d is not a multiple of 128", a->dst_offset);
-        if (a->dst_offset + a->n_tokens > a->cache_tokens)
-            return fail(BITDECODE_EINVAL, "dst_offset %d + n_tokens %d exceeds cache capacity %d", a->dst_offset,
-                        a->n_tokens, a->cache_tokens);
-    } else if (a->n_tokens > a->cache_tokens) {
-        return fail(BITDECODE_EINVAL, "n_tokens %d exceeds cache capacity %d", a->n_tokens, a->cache_tokens);
+        if (static_cast<int64_t>(a->dst_offset) + a->n_tokens > capacity)
+            return fail(BITDECODE_EINVAL, "dst_offset %d + n_tokens %d exceeds cache capacity %lld", a->dst_offset,
+                        a->n_tokens, static_cast<long long>(capacity));
+    } else if (a->n_tokens > capacity) {
+        return fail(BITDECODE_EINVAL, "n_tokens %d exceeds cache capacity %lld", a->n_tokens,
+                    static_cast<long long>(capacity));
     }
+    if (int rc = check_paging(a->block_table, a->block_table_stride, a->max_pages_per_seq, a->num_pages,
+                              a->cache_tokens, 0))
+        return rc;
     if (a->n_tokens == 0 || a->b == 0) return BITDECODE_OK;
     if (!a->k || !a->v || !a->k_pack || !a->k_params || !a->v_pack || !a->v_params)
         return fail(BITDECODE_EINVAL, "null tensor pointer");
@@ -132,6 +152,8 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     P.dst_offset = a->dst_offset;
     P.dst_offsets = a->dst_offsets;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
+    P.block_table = a->block_table; P.bt_stride = a->block_table_stride;
+    P.chunks_per_page = a->cache_tokens / kChunk;
     hipError_t e = launch_qpack(P, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "qpack launch failed: %s", hipGetErrorString(e));
     return BITDECODE_OK;
@@ -150,7 +172,13 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     const int max_r = a->res_lens ? a->max_res_len : a->res_len;
     if (max_s < 0 || max_r < 0) return fail(BITDECODE_EINVAL, "negative length");
     if (max_s % kChunk) return fail(BITDECODE_EINVAL, "packed length %d is not a multiple of 128", max_s);
-    if (max_s > a->cache_tokens) return fail(BITDECODE_EINVAL, "packed length %d exceeds cache capacity %d", max_s, a->cache_tokens);
+    if (!a->block_table && max_s > a->cache_tokens)
+        return fail(BITDECODE_EINVAL, "packed length %d exceeds cache capacity %d", max_s, a->cache_tokens);
+    if (a->block_table && (a->cache_tokens <= 0 || a->cache_tokens % kChunk))
+        return fail(BITDECODE_EINVAL, "page size %d is not a positive multiple of 128", a->cache_tokens);
+    if (int rc = check_paging(a->block_table, a->block_table_stride, a->max_pages_per_seq, a->num_pages,
+                              a->cache_tokens, max_s))
+        return rc;
     if (max_s > 0 && (a->cache_tokens % kChunk)) return fail(BITDECODE_EINVAL, "cache_tokens must be a multiple of 128");
     if (!a->q || !a->out) return fail(BITDECODE_EINVAL, "q/out is null");
     if (max_s > 0 && (!a->k_pack || !a->k_params || !a->v_pack || !a->v_params))
@@ -201,6 +229,8 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     P.scale_log2 = fabsf(a->softmax_scale) * 1.4426950408889634f;   // decode_api.cpp:128-142
     P.neg_scale = a->softmax_scale < 0.0f;
     P.xcd_remap = (a->b * a->h_k) % 8 == 0 && nsplit > 1;
+    P.block_table = a->block_table; P.bt_stride = a->block_table_stride;
+    P.chunks_per_page = a->block_table ? a->cache_tokens / kChunk : 1;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
     if (nsplit > 1) {
         P.tickets = static_cast<int*>(a->workspace);

@@ -328,9 +328,13 @@ struct UnitAddr {
     const uint8_t* vp;
 };
 template <int BITS, int GS>
-__device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int64_t bh, int u) {
+__device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int bi, int hk, int u) {
     using C = UnitCfg<BITS, GS>;
-    const int ci = u / C::UPC, uic = u % C::UPC;
+    const int uic = u % C::UPC;
+    // region and chunk inside it (a paged cache looks the page up in the block table: a scalar load)
+    const ChunkPlace place = chunk_place(P.block_table, P.bt_stride, P.chunks_per_page, bi, hk, P.hk, u / C::UPC);
+    const int64_t bh = place.region;
+    const int ci = place.chunk;
     UnitAddr<BITS, GS> A;      // wave-uniform: everything here lives in SGPRs
     A.kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
     A.vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
@@ -761,7 +765,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     }
     UnitAddr<BITS, GS> A;
     if (u < u1) {
-        A = unit_addr<BITS, GS>(P, bh, u);
+        A = unit_addr<BITS, GS>(P, bi, hk, u);
         issue_kside<BITS, GS>(A, lane * 16, region_lds, 0);
         issue_vside<BITS, GS>(A, lane * 16, region_lds);
         wait_then_take<C::KSIDE + C::VSIDE>(qa, qb, qa_raw, qb_raw);
@@ -805,7 +809,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
 #endif
         int kslot = 0;
         for (int un = u + NW; un < u1; un += NW) {        // units that have a successor: it is fetched from inside
-            A = unit_addr<BITS, GS>(P, bh, un);
+            A = unit_addr<BITS, GS>(P, bi, hk, un);
             compute_unit<BITS, GS, BF16, true>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
             kslot ^= 1;
             phase_ts = nullptr;

@@ -18,6 +18,9 @@ struct QpackParams {
     int dst_offset;
     const int* dst_offsets;
     int bits, gs, bf16;
+    const int* block_table;     // paged cache: page of (sequence, page slot); regions are then (page, kv-head)
+    int64_t bt_stride;
+    int chunks_per_page;
 };
 
 struct FwdParams {
@@ -45,6 +48,9 @@ struct FwdParams {
     int xcd_remap;             // (b * hk) % 8 == 0: keep the splits of one (batch, kv-head) on one XCD
     int neg_scale;             // softmax_scale < 0: the sign is folded into q
     int bits, gs, bf16;
+    const int* block_table;     // paged cache, as in QpackParams
+    int64_t bt_stride;
+    int chunks_per_page;
 };
 
 hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);

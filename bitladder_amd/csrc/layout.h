@@ -36,6 +36,7 @@
 // V params: per chunk 4 sub-blocks x ncg channel groups x 128 B: scale[q][i] (64 B) then
 //   zero[q][i] (64 B), q = 0..3, i = 0..7, token 32*sb + 16*(i/4) + 4*q + i%4.
 #pragma once
+#include <hip/hip_runtime.h>
 #include <stdint.h>
 
 namespace bitdecode {
@@ -54,6 +55,21 @@ constexpr int v_param_chunk_bytes(int gs) { return kChunk * (kHeadDim / gs) * 4;
 constexpr int64_t code_region_bytes(int64_t S, int bits) { return S * kHeadDim * bits / 8; }
 constexpr int64_t k_param_region_bytes(int64_t S, int gs) { return (S / gs) * kKParamGroupBytes; }
 constexpr int64_t v_param_region_bytes(int64_t S, int gs) { return S * (kHeadDim / gs) * 4; }
+
+// Region and chunk-in-region of chunk `ci` of sequence `bi`, kv-head `hk`.  Contiguous cache: region
+// bi * h_k + hk holds all chunks of the sequence.  Paged cache: the block table names the page of every
+// `chunks_per_page` chunks and regions are (page, kv-head).
+struct ChunkPlace {
+    int64_t region;
+    int chunk;
+};
+__host__ __device__ inline ChunkPlace chunk_place(const int* block_table, int64_t bt_stride, int chunks_per_page,
+                                                  int bi, int hk, int n_heads_k, int ci) {
+    if (!block_table) return ChunkPlace{static_cast<int64_t>(bi) * n_heads_k + hk, ci};
+    const int slot = ci / chunks_per_page;
+    const int page = block_table[bi * bt_stride + slot];
+    return ChunkPlace{static_cast<int64_t>(page) * n_heads_k + hk, ci - slot * chunks_per_page};
+}
 
 // ---- decode work units (shared by the kernel and the host-side split choice)
 // A decode wave streams units of 4 KB of K codes + 4 KB of V codes + their parameters through its

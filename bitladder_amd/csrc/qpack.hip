@@ -93,8 +93,9 @@ __global__ __launch_bounds__(256) void qpack_kernel(QpackParams P) {
     const int dst_base = P.dst_offsets ? P.dst_offsets[bi] : P.dst_offset;
     if (dst_base < 0) return;       // a negative per-sequence offset skips that sequence (whole workgroup)
     const int dst_tok = dst_base + ci_src * kChunk;
-    const int ci = dst_tok / kChunk;
-    const int64_t bh = static_cast<int64_t>(bi) * P.hk + hk;
+    const ChunkPlace place = chunk_place(P.block_table, P.bt_stride, P.chunks_per_page, bi, hk, P.hk, dst_tok / kChunk);
+    const int ci = place.chunk;
+    const int64_t bh = place.region;
 
     // ---- global loads of both tiles: thread -> row tid/16 + 16*x, 16-byte column block tid%16
     const int lrow = tid >> 4, lcol = (tid & 15) * 8;

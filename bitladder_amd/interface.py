@@ -35,6 +35,26 @@ def _check_quant(quant_mode: str, group_size: int, num_bits: int) -> None:
         raise ValueError(f"group_size must be 32, 64 or 128, got {group_size}")
 
 
+def _check_block_table(block_table, b, device):
+    """Paged cache (decode_api.cpp:328-335): int32 [batch, max_pages_per_seq], last dim contiguous."""
+    if block_table.dtype != torch.int32:
+        raise RuntimeError("block_table must have dtype torch.int32")
+    if block_table.dim() != 2 or block_table.shape[0] != b:
+        raise RuntimeError("block_table must be [batch, max_pages_per_seq]")
+    if block_table.stride(-1) != 1:
+        raise RuntimeError("block_table must have contiguous last dimension")
+    if block_table.device != device:
+        raise RuntimeError(f"block_table must be on {device}")
+    return block_table
+
+
+def _set_paging(a, block_table, num_pages):
+    a.block_table = block_table.data_ptr()
+    a.block_table_stride = block_table.stride(0)
+    a.max_pages_per_seq = block_table.shape[1]
+    a.num_pages = num_pages
+
+
 def _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device):
     """Validates the caller-allocated packed tensors (evaluation/test.py:74-83) and returns
     (batch, capacity_tokens, h_k)."""
@@ -99,8 +119,6 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     the n new tokens are written, so a full fp16 residual block can be appended to the cache.
     """
     _check_quant(quant_mode, group_size, num_bits)
-    if opt_block_table is not None:
-        raise NotImplementedError("paged KV cache (opt_block_table) is not supported")
     if k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
         raise RuntimeError("k_cache and v_cache must both be [batch, seqlen, nheads_k, head_dim]")
     if not k_cache.is_cuda:
@@ -111,7 +129,10 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     device = k_cache.device
     b, n, h_k, d = k_cache.shape
     cb, S, ch_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device)
-    if (cb, ch_k) != (b, h_k) or d != 128:
+    paged = opt_block_table is not None
+    if paged:      # the cache tensors are page pools: leading dimension = pages, S = page size
+        _check_block_table(opt_block_table, b, device)
+    if (not paged and cb != b) or ch_k != h_k or d != 128:
         raise RuntimeError("packed cache shape does not match k_cache")
     if cu_seqlens_k is not None:
         if cu_seqlens_k.dtype != torch.int32:
@@ -135,6 +156,8 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     a.dst_offset = int(dst_offset)
     a.dst_offsets = None if dst_offsets is None else _i32_dev(dst_offsets, b, device, "dst_offsets").data_ptr()
     a.bits, a.group_size, a.dtype = num_bits, group_size, dtype
+    if paged:
+        _set_paging(a, opt_block_table, cb)
     with torch.cuda.device(device):
         _lib.check(_lib.lib().bitdecode_qpack(ctypes.byref(a), _stream_ptr(device)))
 
@@ -184,8 +207,6 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
                          return_lse: bool = False) -> DecodePlan:
     """Validates a decode call and returns a `DecodePlan`; see `fwd_kvcache_int`."""
     _check_quant(quant_mode, group_size, num_bits)
-    if opt_block_table is not None:
-        raise NotImplementedError("paged KV cache (opt_block_table) is not supported")
     if q.dim() != 4 or q.shape[1] != 1:
         raise RuntimeError("q must be [batch, 1, nheads, head_dim] (one query token per sequence)")
     if not q.is_cuda:
@@ -194,7 +215,10 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
     device = q.device
     b, _, h, d = q.shape
     cb, S, h_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device)
-    if cb != b:
+    paged = opt_block_table is not None
+    if paged:      # page pools: cb pages of S tokens; a sequence holds up to max_pages_per_seq * S tokens
+        _check_block_table(opt_block_table, b, device)
+    elif cb != b:
         raise RuntimeError(f"batch size of q ({b}) and of the packed cache ({cb}) differ")
     if d != 128:
         raise RuntimeError("head dimension must be 128")
@@ -209,12 +233,17 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
     a.k_pack, a.k_params = k_pack.data_ptr(), k_params.data_ptr()
     a.v_pack, a.v_params = v_pack.data_ptr(), v_params.data_ptr()
     a.cache_tokens = S
-    a.seqlen_k = S if seqlen_k is None else int(seqlen_k)
+    capacity = S
+    if paged:
+        keep.append(opt_block_table)
+        _set_paging(a, opt_block_table, cb)
+        capacity = opt_block_table.shape[1] * S        # as the reference: seqlen_k = pages per sequence * page size
+    a.seqlen_k = capacity if seqlen_k is None else int(seqlen_k)
     a.max_seqlen_k = a.seqlen_k
     if seqlens_k is not None:
         keep.append(_i32_dev(seqlens_k, b, device, "seqlens_k"))
         a.seqlens_k = seqlens_k.data_ptr()
-        a.max_seqlen_k = S if max_seqlen_k is None else int(max_seqlen_k)
+        a.max_seqlen_k = capacity if max_seqlen_k is None else int(max_seqlen_k)
     if (k_residual is None) != (v_residual is None):
         raise RuntimeError("k_residual and v_residual must be given together")
     if k_residual is not None:

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define BITDECODE_ABI_VERSION 1
+#define BITDECODE_ABI_VERSION 2
 
 enum {
     BITDECODE_OK = 0,
@@ -55,6 +55,14 @@ typedef struct bitdecode_qpack_args {
     int32_t bits;              /* 2 or 4                                                    */
     int32_t group_size;        /* 32, 64 or 128                                             */
     int32_t dtype;             /* BITDECODE_FP16 / BITDECODE_BF16                           */
+    /* paged cache (csrc/bit_decode/decode_api.cpp:328-352, 420-425): with block_table set, the
+     * four cache tensors are pools of pages, cache_tokens is the page size in tokens (a multiple
+     * of 128) and token t of sequence i lives in page block_table[i * stride + t / cache_tokens].
+     * Entries must lie in [0, num_pages): they are device data and are not checked. */
+    const int32_t* block_table;/* optional device int32[b, max_pages_per_seq]               */
+    int64_t block_table_stride;/* elements between the rows of two sequences                */
+    int32_t max_pages_per_seq; /* columns of block_table                                    */
+    int32_t num_pages;         /* pages in the pool (leading dimension of the cache)        */
 } bitdecode_qpack_args;
 
 int bitdecode_qpack(const bitdecode_qpack_args* args, void* stream);
@@ -92,6 +100,11 @@ typedef struct bitdecode_fwd_args {
     int32_t bits, group_size, dtype;
     float softmax_scale;
     int32_t num_splits;        /* 0 = choose (bitdecode_num_splits); at most 512            */
+    /* paged cache, as in bitdecode_qpack_args: cache_tokens is then the page size */
+    const int32_t* block_table;
+    int64_t block_table_stride;
+    int32_t max_pages_per_seq;
+    int32_t num_pages;
 } bitdecode_fwd_args;
 
 int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);

@@ -225,7 +225,7 @@ def test_python_entry_points_validate_before_touching_the_gpu():
         kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-channel", 48, 4)
     with pytest.raises(ValueError):
         fwd_kvcache_int(t[:, :1], kp, kp, kp, kp, None, 1.0, "k-channel", 128, 3)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError):      # a block table is accepted, but like everything else not on the CPU
         fwd_kvcache_int(t[:, :1], kp, kp, kp, kp, torch.zeros(1, 1, dtype=torch.int32))
     with pytest.raises(RuntimeError):      # CPU tensors: the reference's CHECK_DEVICE
         kvcache_pack_int(t, kp, kp, t, kp, kp)
