@@ -256,6 +256,24 @@ __device__ __forceinline__ void dma_row(const uint8_t* base, uint32_t lane16, ui
                  : "memory", "m0");
 }
 
+// The same with only the first LANES lanes taking part, for a last row that is not full.  The lane
+// mask goes into EXEC around the load inside one asm block (SALU moves only): a branch around the
+// load would split the basic block the scheduler works in.
+template <int OFFSET, int LANES>
+__device__ __forceinline__ void dma_row_first_lanes(const uint8_t* base, uint32_t lane16, uint32_t lds_base) {
+    static_assert(OFFSET >= 0 && OFFSET < 4096 && LANES > 0 && LANES < 64, "immediate offset field, partial row");
+    const uint64_t mask = (1ull << LANES) - 1;
+    uint64_t saved;
+    asm volatile("s_mov_b32 m0, %3\n\t"
+                 "s_mov_b64 %0, exec\n\t"
+                 "s_and_b64 exec, exec, %5\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:%4\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "v"(lane16), "s"(base), "s"(lds_base), "n"(OFFSET), "s"(mask)
+                 : "memory", "m0", "scc");
+}
+
 // s_waitcnt vmcnt(n): at most n of this wave's loads still in flight.  The compiler does not
 // track the asm loads above, so the waits are explicit; the memory clobber keeps LDS reads below.
 template <int N>
@@ -344,13 +362,17 @@ __device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int 
     return A;
 }
 // BYTES contiguous bytes (a multiple of 256) into LDS: whole 1 KB rows, the last one with only the
-// lanes that still have data.  Lane 0 always takes part, so every wave executes every instruction
-// and the vmcnt bookkeeping below holds.
+// first lanes, those that still have data.  Every wave executes every instruction, so the vmcnt
+// bookkeeping below holds.
 template <int BYTES, int R = 0>
 __device__ __forceinline__ void dma_bytes(const uint8_t* src, uint32_t lane16, uint32_t lds_dst) {
     if constexpr (R * 1024 < BYTES) {
         constexpr int left = BYTES - R * 1024;
-        if (left >= 1024 || lane16 < left) dma_row<R * 1024>(src, lane16, lds_dst);
+        if constexpr (left >= 1024) {
+            dma_row<R * 1024>(src, lane16, lds_dst);
+        } else {
+            dma_row_first_lanes<R * 1024, left / 16>(src, lane16, lds_dst);
+        }
         dma_bytes<BYTES, R + 1>(src, lane16, lds_dst);
     }
 }
