@@ -148,6 +148,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fp16", action="store_true", help="skip the fp16-KV baseline leg")
     ap.add_argument("--no-qpack", action="store_true", help="skip the quantize-pack kernel leg")
+    ap.add_argument("--no-step", action="store_true", help="skip the decode-step-with-append leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three plain 256 MiB device copies (a kernel of known traffic, used to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -160,7 +161,7 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
 
-    from bitladder_amd import kvcache_pack_int, plan_fwd_kvcache_int
+    from bitladder_amd import kvcache_pack_int, plan_fwd_kvcache_int, plan_fwd_kvcache_int_append
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -264,6 +265,27 @@ def main():
             "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
             "append_128_tokens_us_per_call": round(us_app, 3)}
         srcs.clear()
+
+    if not args.no_step:
+        # the same decode as one launch that also appends the step's new token (device-side lengths).  A slot
+        # is a packed cache with a window and a length counter of its own, starting at S packed tokens + 64 in
+        # the window; there are enough slots that none sees 60 steps (warm-up, the untimed first replay and
+        # the timed replay together), so no window fills inside the measurement
+        n_slots = max(nbuf, math.ceil((2 * args.steps + args.warmup) / 59))
+        splans = []
+        for i in range(n_slots):
+            cache, kres, vres = keep[i % nbuf]
+            lengths = torch.full((b,), S + 64, dtype=torch.int32, device=dev)
+            q_t = torch.randn((b, 1, h, 128), device=dev).to(dtype)
+            kn = torch.randn((b, 1, h_k, 128), device=dev).to(dtype)
+            splans.append(plan_fwd_kvcache_int_append(q_t, kn, kn.clone(), *cache, kres.clone(), vres.clone(), lengths,
+                                                      S + 127, None, scale, "k-channel", gs, bits,
+                                                      num_splits=args.num_splits))
+        _, est, _ = time_steps(lambda i: splans[i % n_slots].run(), args.steps, args.warmup, not args.no_graph)
+        result["decode_step_with_append"] = {
+            "entry": "bitdecode_fwd_append", "us_per_step": round(est / args.steps * 1e6, 3),
+            "window_tokens": "65-123", "does": "attend + store the new token + advance the device-side length"}
+        del splans
 
     if not args.no_fp16:
         # fp16-KV decode on the same GPU: the library's own fp16 split-KV path over all S+R tokens,

@@ -7,7 +7,9 @@ __version__ = "1.0.0.post1"
 from .interface import (  # noqa: F401
     DecodePlan,
     fwd_kvcache_int,
+    fwd_kvcache_int_append,
     kvcache_pack_int,
     plan_fwd_kvcache_int,
+    plan_fwd_kvcache_int_append,
 )
 from .cache import BitKVCache  # noqa: F401,E402

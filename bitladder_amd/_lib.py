@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbitdecode.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 FP16, BF16 = 0, 1
 
 _i32, _i64, _vp, _f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
@@ -55,8 +55,20 @@ class FwdArgs(ctypes.Structure):
     ]
 
 
+class FwdAppendArgs(ctypes.Structure):
+    _fields_ = [
+        ("fwd", FwdArgs),
+        ("lengths", _vp),
+        ("k_new", _vp), ("v_new", _vp),
+        ("knew_stride_b", _i64), ("knew_stride_h", _i64),
+        ("vnew_stride_b", _i64), ("vnew_stride_h", _i64),
+        ("max_len", _i32),
+    ]
+
+
 EXPORTS = ("bitdecode_abi_version", "bitdecode_last_error", "bitdecode_num_splits",
-           "bitdecode_fwd_workspace_bytes", "bitdecode_qpack", "bitdecode_fwd")
+           "bitdecode_fwd_workspace_bytes", "bitdecode_qpack", "bitdecode_fwd",
+           "bitdecode_fwd_append", "bitdecode_fwd_append_workspace_bytes")
 
 _lib = None
 
@@ -89,6 +101,10 @@ def lib():
         L.bitdecode_qpack.argtypes = [ctypes.POINTER(QpackArgs), _vp]
         L.bitdecode_fwd.restype = ctypes.c_int
         L.bitdecode_fwd.argtypes = [ctypes.POINTER(FwdArgs), _vp]
+        L.bitdecode_fwd_append.restype = ctypes.c_int
+        L.bitdecode_fwd_append.argtypes = [ctypes.POINTER(FwdAppendArgs), _vp]
+        L.bitdecode_fwd_append_workspace_bytes.restype = ctypes.c_size_t
+        L.bitdecode_fwd_append_workspace_bytes.argtypes = [_i32] * 3
         if L.bitdecode_abi_version() != ABI_VERSION:
             raise ImportError("libbitdecode.so ABI version mismatch; rebuild it")
         _lib = L

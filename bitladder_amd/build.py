@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -13,13 +14,15 @@ LIB_PATH = os.path.join(_HERE, "libbitdecode.so")
 ARCH = "gfx950"
 COMMON = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
           # packed-FP32 VALU forms are kept out of the generated code on purpose
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          # per-kernel register / scratch report, checked below
+          "-Rpass-analysis=kernel-resource-usage"]
 # the quantizer must be IEEE fp32: no contraction, correctly rounded division;
 # the decode kernel is scheduled for instruction-level parallelism rather than for occupancy (its
 # occupancy is fixed by LDS): 2-3 % faster on the long-context workloads, same register counts
 PER_FILE = {
     "qpack.hip": ["-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"],
-    "decode.hip": ["-mllvm", "-amdgpu-sched-strategy=gcn-max-ilp"],
+    "decode.hip": ["-mllvm", "-amdgpu-sched-strategy=gcn-max-ilp", "-fhip-fp32-correctly-rounded-divide-sqrt"],
     "api.hip": [],
 }
 
@@ -29,6 +32,19 @@ def hipcc() -> str:
     if not os.path.exists(exe):
         raise RuntimeError("hipcc not found")
     return exe
+
+
+def check_no_scratch(src: str, report: str) -> None:
+    """No kernel of the library may spill registers: a kernel with a scratch segment pays for its set-up
+    at every launch (about 1 us on the decode kernel), whether or not the spilling path runs."""
+    name = None
+    for line in report.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and int(m.group(1)) > 0:
+            raise RuntimeError(f"{src}: kernel {name} needs {m.group(1)} bytes of scratch per lane (register spills)")
 
 
 def build(verbose: bool = False) -> str:
@@ -49,6 +65,7 @@ def build(verbose: bool = False) -> str:
         out, _ = p.communicate()
         if p.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+        check_no_scratch(src, out)
     cmd = [cc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:

@@ -6,8 +6,10 @@ recent `L mod N_r` tokens stay fp16 and are attended in fp16; when the window re
 quantize-packed and appended to the cache) and that its kernel traits still name
 (csrc/bit_decode/src/include/kernel_traits.h:76,85: residual_block_size).  The reference's main branch
 ships no code for it; here it is host logic over `kvcache_pack_int(dst_offsets=...)` and
-`fwd_kvcache_int(seqlens_k=..., residual_len=...)`.  Lengths are tracked on the host (they are a pure
-function of the calls made), so nothing is read back from the device.
+`fwd_kvcache_int(seqlens_k=..., residual_len=...)`, or one launch per token with
+`fwd_kvcache_int_append` (`step`).  Lengths are tracked on the host (they are a pure function of the
+calls made) and mirrored in a device counter that `step` advances, so nothing is read back from the
+device.
 """
 from __future__ import annotations
 
@@ -16,7 +18,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from .interface import fwd_kvcache_int, kvcache_pack_int
+from .interface import fwd_kvcache_int, kvcache_pack_int, plan_fwd_kvcache_int_append
 
 BLOCK = 128          # tokens per packed block = residual window size N_r
 
@@ -46,6 +48,7 @@ class BitKVCache:
         self.v_res = torch.zeros_like(self.k_res)
         self.packed_len = [0] * batch
         self.res_len = [0] * batch
+        self.total = torch.zeros(batch, dtype=torch.int32, device=dev)     # tokens held, as `step` needs them
         self._rows = torch.arange(batch, device=dev)
 
     # ------------------------------------------------------------------ lengths
@@ -79,6 +82,7 @@ class BitKVCache:
             if r:
                 self.k_res[i, :r].copy_(k[i, p:p + r])
                 self.v_res[i, :r].copy_(v[i, p:p + r])
+        self.total.copy_(self._i32(lengths))
 
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:
         """Append one token per sequence, `[b, 1, h_k, 128]` (or `[b, h_k, 128]`).  A window that reaches 128
@@ -99,6 +103,7 @@ class BitKVCache:
                              None, None, BLOCK, "k-channel", self.gs, self.bits, dst_offsets=offsets)
             self.packed_len = [p + BLOCK if f else p for p, f in zip(self.packed_len, full)]
             self.res_len = [0 if f else r for r, f in zip(self.res_len, full)]
+        self.total += 1
 
     # ------------------------------------------------------------------ read
     def decode(self, q: torch.Tensor, softmax_scale: Optional[float] = None, **kw) -> torch.Tensor:
@@ -111,3 +116,43 @@ class BitKVCache:
                                seqlens_k=self._i32(self.packed_len), max_seqlen_k=max_p,
                                k_residual=self.k_res, v_residual=self.v_res,
                                residual_len=self._i32(self.res_len), max_residual_len=max_r, **kw)
+
+    # ------------------------------------------------------------------ one launch per token
+    def plan_step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                  softmax_scale: Optional[float] = None, **kw):
+        """A `DecodePlan` whose `run()` is one decode step in one launch: attend `q` over everything held
+        plus the new token, append the token, pack the window if it became full.  The plan reads
+        `q / k_new / v_new` in place and sizes its grid for the cache's capacity, so it can be run (or
+        captured in a HIP graph and replayed) once per token.  Lengths advance on the device; the host
+        copies do not follow a plan that is run directly: call `sync_lengths()` before mixing it with the
+        other methods."""
+        if softmax_scale is None:
+            softmax_scale = 1.0 / math.sqrt(q.shape[-1])
+        return plan_fwd_kvcache_int_append(q, k_new, v_new, self.k_pack, self.k_params, self.v_pack, self.v_params,
+                                           self.k_res, self.v_res, self.total, self.capacity + BLOCK - 1, None,
+                                           softmax_scale, "k-channel", self.gs, self.bits, **kw)
+
+    def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+             softmax_scale: Optional[float] = None, **kw) -> torch.Tensor:
+        """`append` and `decode` in one launch, except that a window filled by this token is attended in
+        fp16 once more before its packed form takes over.  A sequence that has no room left is attended
+        but not extended."""
+        if k_new.dim() == 3:
+            k_new, v_new = k_new[:, None], v_new[:, None]
+        if any(p + r + 1 > self.capacity for p, r in zip(self.packed_len, self.res_len)):
+            raise ValueError("step: cache capacity exceeded")
+        plan = self.plan_step(q, k_new.to(self.dtype), v_new.to(self.dtype), softmax_scale, **kw)
+        with torch.cuda.device(self.device):
+            out = plan.run()
+        for i, (p, r) in enumerate(zip(self.packed_len, self.res_len)):
+            if r + 1 < BLOCK:
+                self.res_len[i] = r + 1
+            elif p + BLOCK <= self.capacity:
+                self.packed_len[i], self.res_len[i] = p + BLOCK, 0
+        return out
+
+    def sync_lengths(self) -> None:
+        """Reads the device counter back (synchronises) and rebuilds the host copies from it."""
+        totals = self.total.tolist()
+        self.packed_len = [t // BLOCK * BLOCK for t in totals]
+        self.res_len = [t - p for t, p in zip(totals, self.packed_len)]

@@ -159,7 +159,15 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     return BITDECODE_OK;
 }
 
-int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
+// bytes of the per-sequence step counters that lead a step workspace
+static size_t step_ticket_bytes(int32_t b) { return (static_cast<size_t>(b) * sizeof(int) + 255) / 256 * 256; }
+
+size_t bitdecode_fwd_append_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
+    return step_ticket_bytes(b) + bitdecode_fwd_workspace_bytes(b, h, num_splits);
+}
+
+// decode, or (step != null) decode step with append
+static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args* step, void* stream) {
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
     if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
@@ -168,8 +176,25 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     const int g = a->h / a->h_k;
     if (g > kMaxGroupHeads)
         return fail(BITDECODE_EUNSUPPORTED, "%d query heads per kv head unsupported (at most %d)", g, kMaxGroupHeads);
-    const int max_s = a->seqlens_k ? a->max_seqlen_k : a->seqlen_k;
-    const int max_r = a->res_lens ? a->max_res_len : a->res_len;
+    int max_s = a->seqlens_k ? a->max_seqlen_k : a->seqlen_k;
+    int max_r = a->res_lens ? a->max_res_len : a->res_len;
+    if (step) {
+        // lengths live on the device; the host bound sizes the grid: up to max_len tokens before the
+        // step, of which whole chunks are packed, and a window of up to 128 tokens with the new one
+        if (!step->lengths || !step->k_new || !step->v_new)
+            return fail(BITDECODE_EINVAL, "decode step: lengths, k_new and v_new are required");
+        if (step->max_len < 0) return fail(BITDECODE_EINVAL, "decode step: max_len %d is negative", step->max_len);
+        if (!a->k_res || !a->v_res || a->max_res_len < kChunk)
+            return fail(BITDECODE_EINVAL, "decode step: a residual window of at least 128 tokens is required "
+                                          "(max_res_len = its capacity, got %d)", a->max_res_len);
+        if (!aligned16(step->k_new) || !aligned16(step->v_new))
+            return fail(BITDECODE_EINVAL, "tensor pointers must be 16-byte aligned");
+        const int64_t ns[4] = {step->knew_stride_b, step->knew_stride_h, step->vnew_stride_b, step->vnew_stride_h};
+        for (int64_t s : ns)
+            if (s % 8) return fail(BITDECODE_EINVAL, "k_new / v_new strides must be multiples of 8 elements");
+        max_s = step->max_len / kChunk * kChunk;
+        max_r = kChunk;
+    }
     if (max_s < 0 || max_r < 0) return fail(BITDECODE_EINVAL, "negative length");
     if (max_s % kChunk) return fail(BITDECODE_EINVAL, "packed length %d is not a multiple of 128", max_s);
     if (!a->block_table && max_s > a->cache_tokens)
@@ -181,8 +206,10 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
         return rc;
     if (max_s > 0 && (a->cache_tokens % kChunk)) return fail(BITDECODE_EINVAL, "cache_tokens must be a multiple of 128");
     if (!a->q || !a->out) return fail(BITDECODE_EINVAL, "q/out is null");
-    if (max_s > 0 && (!a->k_pack || !a->k_params || !a->v_pack || !a->v_params))
+    if ((max_s > 0 || step) && (!a->k_pack || !a->k_params || !a->v_pack || !a->v_params))
         return fail(BITDECODE_EINVAL, "null packed-cache pointer");
+    if (step && (a->cache_tokens <= 0 || a->cache_tokens % kChunk))
+        return fail(BITDECODE_EINVAL, "cache_tokens %d is not a positive multiple of 128", a->cache_tokens);
     if (max_r > 0 && (!a->k_res || !a->v_res)) return fail(BITDECODE_EINVAL, "null residual pointer");
     if (!aligned16(a->q) || !aligned16(a->k_pack) || !aligned16(a->k_params) || !aligned16(a->v_pack) ||
         !aligned16(a->v_params) || !aligned16(a->k_res) || !aligned16(a->v_res))
@@ -196,8 +223,9 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
     if (nsplit > 512) return fail(BITDECODE_EINVAL, "num_splits %d is above the limit of 512", nsplit);
     if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
-    if (nsplit > 1) {
-        const size_t need = bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
+    if (nsplit > 1 || step) {
+        const size_t need = step ? bitdecode_fwd_append_workspace_bytes(a->b, a->h, nsplit)
+                                 : bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
         if (!a->workspace || a->workspace_bytes < need)
             return fail(BITDECODE_EWORKSPACE, "workspace of %zu bytes needed for %d splits, got %zu", need, nsplit,
                         a->workspace ? a->workspace_bytes : size_t(0));
@@ -232,14 +260,33 @@ int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) {
     P.block_table = a->block_table; P.bt_stride = a->block_table_stride;
     P.chunks_per_page = a->block_table ? a->cache_tokens / kChunk : 1;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    if (step) {
+        P.lengths = step->lengths;
+        P.step_tickets = reinterpret_cast<int*>(ws);
+        ws += step_ticket_bytes(a->b);
+        P.k_new = static_cast<const uint16_t*>(step->k_new);
+        P.v_new = static_cast<const uint16_t*>(step->v_new);
+        P.knew_sb = step->knew_stride_b; P.knew_sh = step->knew_stride_h;
+        P.vnew_sb = step->vnew_stride_b; P.vnew_sh = step->vnew_stride_h;
+        const int64_t cap = a->block_table ? static_cast<int64_t>(a->max_pages_per_seq) * a->cache_tokens : a->cache_tokens;
+        P.capacity = static_cast<int>(std::min<int64_t>(cap, INT32_MAX / 2));
+    }
     if (nsplit > 1) {
-        P.tickets = static_cast<int*>(a->workspace);
-        P.o_part = reinterpret_cast<float*>(static_cast<uint8_t*>(a->workspace) + ticket_bytes(a->b, a->h));
+        P.tickets = reinterpret_cast<int*>(ws);
+        P.o_part = reinterpret_cast<float*>(ws + ticket_bytes(a->b, a->h));
         P.ml_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
     }
     hipError_t e = launch_fwd(P, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));
     return BITDECODE_OK;
+}
+
+int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) { return run_fwd(a, nullptr, stream); }
+
+int bitdecode_fwd_append(const bitdecode_fwd_append_args* a, void* stream) {
+    if (!a) return fail(BITDECODE_EINVAL, "args is null");
+    return run_fwd(&a->fwd, a, stream);
 }
 
 #ifdef BITDECODE_PROF

@@ -37,10 +37,12 @@
 //    workgroup publishes its unnormalised (O, max, sum) and the one that draws the last ticket
 //    of a (batch, kv-head) combines all of them.
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "kernels.h"
 #include "layout.h"
+#include "qpack_chunk.h"
 
 namespace bitdecode {
 namespace {
@@ -564,6 +566,53 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     PHASE(15);
 }
 
+// Fields of the kernel's parameter block, re-read from the kernarg segment at the point of use.  The
+// fields that only the append needs would otherwise sit in scalar registers through the whole kernel
+// (the compiler loads every kernel argument up front), and the unit loop has none to spare: they get
+// spilled to vector-register lanes inside it.  Scalar loads, written out so that they stay where they
+// are; the kernel's only argument is the FwdParams block, at offset 0 of the segment.
+template <int OFF>
+__device__ __forceinline__ uint32_t karg_u32() {
+    uint32_t v;
+    asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                 : "=s"(v) : "s"(__builtin_amdgcn_kernarg_segment_ptr()), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF>
+__device__ __forceinline__ uint64_t karg_u64() {
+    uint64_t v;
+    asm volatile("s_load_dwordx2 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                 : "=s"(v) : "s"(__builtin_amdgcn_kernarg_segment_ptr()), "n"(OFF) : "memory");
+    return v;
+}
+// sixteen consecutive dwords in one load, and a field picked out of them
+typedef uint32_t kblock __attribute__((ext_vector_type(16)));
+template <int OFF>
+__device__ __forceinline__ kblock karg_block() {
+    static_assert(OFF % 4 == 0 && OFF + 64 <= static_cast<int>(sizeof(FwdParams)), "inside the parameter block");
+    kblock v;
+    asm volatile("s_load_dwordx16 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                 : "=s"(v) : "s"(__builtin_amdgcn_kernarg_segment_ptr()), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF, int FIELD_OFF>
+__device__ __forceinline__ uint64_t block_u64(const kblock& v) {
+    static_assert(FIELD_OFF >= OFF && FIELD_OFF + 8 <= OFF + 64 && (FIELD_OFF - OFF) % 4 == 0, "field inside the block");
+    return v[(FIELD_OFF - OFF) / 4] | (static_cast<uint64_t>(v[(FIELD_OFF - OFF) / 4 + 1]) << 32);
+}
+template <int OFF, int FIELD_OFF>
+__device__ __forceinline__ uint32_t block_u32(const kblock& v) {
+    static_assert(FIELD_OFF >= OFF && FIELD_OFF + 4 <= OFF + 64 && (FIELD_OFF - OFF) % 4 == 0, "field inside the block");
+    return v[(FIELD_OFF - OFF) / 4];
+}
+#define BLOCK_AT(field) offsetof(FwdParams, field)
+#define BLOCK_PTR(type, blk, first, field) reinterpret_cast<type>(block_u64<BLOCK_AT(first), BLOCK_AT(field)>(blk))
+#define BLOCK_I64(blk, first, field) static_cast<int64_t>(block_u64<BLOCK_AT(first), BLOCK_AT(field)>(blk))
+#define BLOCK_I32(blk, first, field) static_cast<int>(block_u32<BLOCK_AT(first), BLOCK_AT(field)>(blk))
+#define LATE_I32(field) static_cast<int>(karg_u32<offsetof(FwdParams, field)>())
+#define LATE_I64(field) static_cast<int64_t>(karg_u64<offsetof(FwdParams, field)>())
+#define LATE_PTR(type, field) reinterpret_cast<type>(karg_u64<offsetof(FwdParams, field)>())
+
 // ---------------------------------------------------------------------------------------------
 // 16-token tiles of the fp16 residual window (tokens n0 .. n0+15, valid below R)
 // ---------------------------------------------------------------------------------------------
@@ -572,22 +621,56 @@ struct Fp16Tile {
     u4 v[4];   // lane (kg, col): token 4*x + kg, channels 8*col .. +7
 };
 
-__device__ __forceinline__ void load_fp16_tile(Fp16Tile& T, const FwdParams& P, int bi, int hk, int n0, int R,
-                                               int lane) {
+// Where the window's rows are, for one (batch, kv-head).  With APPEND the window's row r_new is not in
+// the window yet: it is the step's new token (kn, vn).
+struct WindowSrc {
+    const uint16_t* kr;
+    const uint16_t* vr;
+    int64_t k_st, v_st;
+    const uint16_t* kn;
+    const uint16_t* vn;
+};
+template <bool APPEND>
+__device__ __forceinline__ WindowSrc window_src(const FwdParams& P, int bi, int hk) {
+    WindowSrc W;
+    if constexpr (!APPEND) {
+        W.kr = P.k_res + bi * P.kres_sb + hk * P.kres_sh;
+        W.vr = P.v_res + bi * P.vres_sb + hk * P.vres_sh;
+        W.k_st = P.kres_st;
+        W.v_st = P.vres_st;
+        W.kn = W.vn = nullptr;
+        return W;
+    }
+    // The decode step needs more parameter fields than the scalar registers hold next to the unit loop's
+    // state: what the loop does not use is fetched from the kernarg segment only here.
+    const kblock kb = karg_block<BLOCK_AT(k_res)>();      // k_res ... vres_sh
+    W.kr = BLOCK_PTR(const uint16_t*, kb, k_res, k_res) + bi * BLOCK_I64(kb, k_res, kres_sb) + hk * BLOCK_I64(kb, k_res, kres_sh);
+    W.vr = BLOCK_PTR(const uint16_t*, kb, k_res, v_res) + bi * BLOCK_I64(kb, k_res, vres_sb) + hk * BLOCK_I64(kb, k_res, vres_sh);
+    W.k_st = BLOCK_I64(kb, k_res, kres_st);
+    W.v_st = BLOCK_I64(kb, k_res, vres_st);
+    W.kn = W.vn = nullptr;
+    if constexpr (APPEND) {
+        W.kn = LATE_PTR(const uint16_t*, k_new) + bi * LATE_I64(knew_sb) + hk * LATE_I64(knew_sh);
+        W.vn = LATE_PTR(const uint16_t*, v_new) + bi * LATE_I64(vnew_sb) + hk * LATE_I64(vnew_sh);
+    }
+    return W;
+}
+template <bool APPEND>
+__device__ __forceinline__ void load_fp16_tile(Fp16Tile& T, const WindowSrc& W, int n0, int R, int lane, int r_new) {
     const int col = lane & 15, kg = lane >> 4;
-    const uint16_t* kr = P.k_res + bi * P.kres_sb + hk * P.kres_sh;
-    const uint16_t* vr = P.v_res + bi * P.vres_sb + hk * P.vres_sh;
     const int tok = n0 + col;
+    const uint16_t* krow = (APPEND && tok == r_new) ? W.kn : W.kr + static_cast<int64_t>(tok) * W.k_st;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         T.k[j] = u4{0, 0, 0, 0};
-        if (tok < R) T.k[j] = ld_u4(kr + static_cast<int64_t>(tok) * P.kres_st + 32 * j + 8 * kg);
+        if (tok < R) T.k[j] = ld_u4(krow + 32 * j + 8 * kg);
     }
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
         const int tv = n0 + 4 * x + kg;
+        const uint16_t* vrow = (APPEND && tv == r_new) ? W.vn : W.vr + static_cast<int64_t>(tv) * W.v_st;
         T.v[x] = u4{0, 0, 0, 0};
-        if (tv < R) T.v[x] = ld_u4(vr + static_cast<int64_t>(tv) * P.vres_st + col * 8);
+        if (tv < R) T.v[x] = ld_u4(vrow + col * 8);
     }
 }
 
@@ -703,6 +786,86 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// decode step with append: per-sequence length, the workgroup that stores and packs, the counter
+// ---------------------------------------------------------------------------------------------
+// The length is stable for every workgroup that reads it: it is advanced only after all workgroups of
+// the sequence have drawn their tickets.
+__device__ __forceinline__ int step_length(const FwdParams& P, int bi) { return P.lengths[bi]; }
+// A sequence whose window is about to fill while its cache has no room for another chunk cannot
+// take the token: it is attended, but neither stored nor counted.
+__device__ __forceinline__ bool step_overflows(int capacity, int t) {
+    const int r = t & (kChunk - 1);
+    return t < 0 || (r == kChunk - 1 && t - r + kChunk > capacity);
+}
+// The workgroup that writes the output of a (batch, kv-head) is the last one of that pair to use the
+// length and the window.  One of its threads draws a ticket as soon as that is settled; the holder of
+// the last of the h_k tickets of a sequence knows that every workgroup of the sequence has read the
+// length, advances it and resets the counter.
+__device__ __forceinline__ void step_ticket(int* step_tickets, int* lengths, int n_heads_k, int capacity, int bi, int t) {
+    const int drawn = __hip_atomic_fetch_add(&step_tickets[bi], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (drawn == n_heads_k - 1) {
+        // read again only by the next launch: plain stores
+        step_tickets[bi] = 0;
+        if (!step_overflows(capacity, t)) lengths[bi] = t + 1;
+    }
+}
+
+// Append of one (batch, kv-head) by the workgroup that finishes the pair, in two parts.  Both run after
+// every other workgroup of the pair has finished, so nobody else reads the window any more.
+//
+// First part, as early as that is known, by the two last waves (the waves with the least to do in the
+// merge, so that the round trips below overlap the other waves' work): 32 lanes of the last wave copy
+// the new token into the window's next row, lane 0 of the wave before it sees to the length.
+template <int NW>
+__device__ __forceinline__ void step_begin(int bi, int hk, int t) {
+    static_assert(NW >= 2, "two waves share the append");
+    const int tid = threadIdx.x;
+    const int capacity = LATE_I32(capacity);
+    if (tid == (NW - 2) * 64) {
+        step_ticket(LATE_PTR(int*, step_tickets), LATE_PTR(int*, lengths), LATE_I32(hk), capacity, bi, t);
+    }
+    const int lt = tid - (NW - 1) * 64;
+    if (lt < 0 || lt >= 32 || step_overflows(capacity, t)) return;
+    const int r = t & (kChunk - 1);
+    if (lt < 16) {
+        const uint16_t* kn = LATE_PTR(const uint16_t*, k_new) + bi * LATE_I64(knew_sb) + hk * LATE_I64(knew_sh);
+        uint16_t* kw = LATE_PTR(uint16_t*, k_res) + bi * LATE_I64(kres_sb) + hk * LATE_I64(kres_sh);
+        *reinterpret_cast<u4*>(kw + r * LATE_I64(kres_st) + lt * 8) = ld_u4(kn + lt * 8);
+    } else {
+        const uint16_t* vn = LATE_PTR(const uint16_t*, v_new) + bi * LATE_I64(vnew_sb) + hk * LATE_I64(vnew_sh);
+        uint16_t* vw = LATE_PTR(uint16_t*, v_res) + bi * LATE_I64(vres_sb) + hk * LATE_I64(vres_sh);
+        *reinterpret_cast<u4*>(vw + r * LATE_I64(vres_st) + (lt - 16) * 8) = ld_u4(vn + (lt - 16) * 8);
+    }
+}
+// Second part, by the whole workgroup once the output is written: a window that the token filled is
+// quantize-packed (127 rows from the window, the last one from the new-token tensors) into the chunk
+// behind the packed prefix.  `lds` is the workgroup's whole dynamic LDS.
+template <int BITS, int GS, bool BF16>
+__device__ __forceinline__ void step_end(uint8_t* lds, int bi, int hk, int t) {
+    const int tid = threadIdx.x;
+    const int r = t & (kChunk - 1), packed = t - r;
+    if (__builtin_expect(r == kChunk - 1, 0)) {      // uniform over the workgroup
+        if (step_overflows(LATE_I32(capacity), t)) return;
+        __syncthreads();        // the LDS still holds the merge weights some threads are reading
+        const uint16_t* kn = LATE_PTR(const uint16_t*, k_new) + bi * LATE_I64(knew_sb) + hk * LATE_I64(knew_sh);
+        const uint16_t* vn = LATE_PTR(const uint16_t*, v_new) + bi * LATE_I64(vnew_sb) + hk * LATE_I64(vnew_sh);
+        const uint16_t* kw = LATE_PTR(const uint16_t*, k_res) + bi * LATE_I64(kres_sb) + hk * LATE_I64(kres_sh);
+        const uint16_t* vw = LATE_PTR(const uint16_t*, v_res) + bi * LATE_I64(vres_sb) + hk * LATE_I64(vres_sh);
+        const int64_t k_st = LATE_I64(kres_st), v_st = LATE_I64(vres_st);
+        const ChunkPlace place = chunk_place(LATE_PTR(const int*, block_table), LATE_I64(bt_stride),
+                                             LATE_I32(chunks_per_page), bi, hk, LATE_I32(hk), packed / kChunk);
+        const qp::ChunkDst D = qp::chunk_dst<BITS, GS>(
+            LATE_PTR(uint8_t*, k_pack), LATE_PTR(uint8_t*, k_params), LATE_PTR(uint8_t*, v_pack),
+            LATE_PTR(uint8_t*, v_params), LATE_I64(kpack_bh), LATE_I64(kparams_bh), LATE_I64(vpack_bh),
+            LATE_I64(vparams_bh), place);
+        qp::pack_chunk<BITS, GS, BF16, false>(
+            *reinterpret_cast<qp::PackLds<GS>*>(lds), tid, tid < qp::kPackThreads,
+            [=](int n) { return n == kChunk - 1 ? kn : kw + n * k_st; },
+            [=](int n) { return n == kChunk - 1 ? vn : vw + n * v_st; }, D);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // split-KV kernel: 1-D grid of num_splits * h_k * b workgroups of UnitCfg::NW waves.
 // Split s of a (batch, kv-head) owns packed units [s*ups, (s+1)*ups) dealt round-robin to its
 // waves; the 16-token tiles of the fp16 window are dealt round-robin over ALL waves of the head.
@@ -722,11 +885,12 @@ constexpr int fwd_lds_bytes() {
     return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + (3 * C::NW + 2) * kMaxGroupHeads * 4 + 16;
 }
 
-template <int BITS, int GS, bool BF16>
+template <int BITS, int GS, bool BF16, bool APPEND>
 __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
     using C = UnitCfg<BITS, GS>;
     constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    static_assert(sizeof(qp::PackLds<GS>) <= NW * REGION, "the pack tile reuses the wave regions");
     uint8_t* const sq = lds + NW * REGION;                                   // [8 + zero row][128] 16-bit q
     float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * kQRowBytes);   // [NW][8]
     float* const sL = sM + NW * kMaxGroupHeads;
@@ -762,8 +926,16 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     const int g = P.g;
     const int64_t bh = static_cast<int64_t>(bi) * P.hk + hk;
 
-    const int S = P.seqlens ? P.seqlens[bi] : P.seqlen;
-    const int R = P.reslens ? P.reslens[bi] : P.reslen;
+    int S, R, r_new = -1, step_len = 0;
+    if constexpr (APPEND) {
+        step_len = step_length(P, bi);
+        r_new = step_len & (kChunk - 1);
+        S = min(step_len - r_new, P.capacity);     // a length beyond the capacity is the caller's error: stay inside
+        R = r_new + 1;
+    } else {
+        S = P.seqlens ? P.seqlens[bi] : P.seqlen;
+        R = P.reslens ? P.reslens[bi] : P.reslen;
+    }
     const int nU = (S / kChunk) * C::UPC;
     const int ups = (nU + P.nsplit - 1) / P.nsplit;
     const int u0 = min(nU, split * ups);
@@ -846,14 +1018,15 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         int t = wave * P.nsplit + split;   // consecutive tiles go to different workgroups
         if (t < nT) {
             wait_vm<0>();                  // q rows (a wave without packed units has not waited yet)
+            const WindowSrc W = window_src<APPEND>(P, bi, hk);
             Fp16Tile T;
-            load_fp16_tile(T, P, bi, hk, t * 16, R, lane);
+            load_fp16_tile<APPEND>(T, W, t * 16, R, lane, r_new);
             while (true) {
                 const int tn = t + stride;
                 const bool more = tn < nT;
                 fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, Q, lo_part, st, slab);
                 if (!more) break;
-                load_fp16_tile(T, P, bi, hk, tn * 16, R, lane);
+                load_fp16_tile<APPEND>(T, W, tn * 16, R, lane, r_new);
                 t = tn;
             }
         }
@@ -882,6 +1055,9 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     }
     __syncthreads();
     PROF(4);
+    if constexpr (APPEND) {
+        if (P.nsplit == 1) step_begin<NW>(bi, hk, step_len);     // a single split: every wave is past the window
+    }
     // one wave turns the per-wave maxima and sums into weights: lane (w8, head) covers waves w8, w8 + 8
     if (wave == 0) {
         const int hh = lane & 7, w8 = lane >> 3;
@@ -906,7 +1082,26 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     __syncthreads();
     // the workgroup's result relative to its own maximum: O = sum_w a_w O_w, with (M, L) per head.
     // A single split normalises and writes the output; otherwise the triple is published as is.
-    const int64_t hstride = static_cast<int64_t>(P.b) * P.h;       // rows per split in the workspace
+    uint16_t* out = P.out;
+    int64_t out_sb = P.out_sb, out_sh = P.out_sh;
+    float* lse_out = P.lse;
+    float* o_part = P.o_part;
+    float* ml_part = P.ml_part;
+    int* tickets = P.tickets;
+    int n_h = P.h, n_b = P.b;
+    if constexpr (APPEND) {      // as for the window: fetched late
+        const kblock ob = karg_block<BLOCK_AT(o_part)>();       // o_part ... h
+        out = BLOCK_PTR(uint16_t*, ob, o_part, out);
+        out_sb = BLOCK_I64(ob, o_part, out_sb);
+        out_sh = BLOCK_I64(ob, o_part, out_sh);
+        lse_out = BLOCK_PTR(float*, ob, o_part, lse);
+        o_part = BLOCK_PTR(float*, ob, o_part, o_part);
+        ml_part = BLOCK_PTR(float*, ob, o_part, ml_part);
+        tickets = BLOCK_PTR(int*, ob, o_part, tickets);
+        n_h = BLOCK_I32(ob, o_part, h);
+        n_b = BLOCK_I32(ob, o_part, b);
+    }
+    const int64_t hstride = static_cast<int64_t>(n_b) * n_h;       // rows per split in the workspace
     for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
         const int hh = idx >> 7, c = idx & 127;
         float aw[NW];      // NW is a multiple of 4: four weights per LDS read
@@ -924,26 +1119,22 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         const int hq = hk * g + hh;
         if (P.nsplit == 1) {
             const bool empty = !(L > 0.0f);
-            P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(empty ? 0.0f : O / L);
+            out[bi * out_sb + hq * out_sh + c] = to_out<BF16>(empty ? 0.0f : O / L);
             // natural-log LSE (softmax.h:303); +inf for a row without keys
-            if (c == 0 && P.lse) {
-                P.lse[bi * P.h + hq] = empty ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+            if (c == 0 && lse_out) {
+                lse_out[bi * n_h + hq] = empty ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
             }
         } else {
-            const int64_t row = split * hstride + bi * P.h + hq;
-            st_dev(&P.o_part[row * kHeadDim + c], O);
+            const int64_t row = split * hstride + bi * n_h + hq;
+            st_dev(&o_part[row * kHeadDim + c], O);
             if (c == 0) {
-                st_dev(&P.ml_part[2 * row], M);
-                st_dev(&P.ml_part[2 * row + 1], L);
+                st_dev(&ml_part[2 * row], M);
+                st_dev(&ml_part[2 * row + 1], L);
             }
         }
     }
     PROF(5);
-    if (P.nsplit == 1) {
-        PROF_FLUSH();
-        return;
-    }
-
+    if (P.nsplit > 1) {
     // ---- the workgroup that draws the last ticket of this (batch, kv-head) merges the splits.
     // Partials are written with device-scope (write-through) stores; once a thread's stores have
     // completed (vmcnt 0) and the workgroup has met at the barrier, thread 0 takes the ticket.
@@ -952,10 +1143,10 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     wait_vm<0>();
     __syncthreads();
     if (tid == 0) {
-        const int old = __hip_atomic_fetch_add(&P.tickets[bh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = __hip_atomic_fetch_add(&tickets[bh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const int last = (old == P.nsplit - 1);
         *s_last = last;
-        if (last) __hip_atomic_store(&P.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (last) __hip_atomic_store(&tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     PROF(6);
@@ -963,6 +1154,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         PROF_FLUSH();
         return;
     }
+    if constexpr (APPEND) step_begin<NW>(bi, hk, step_len);     // every other split of the pair has finished
     // Every thread owns one (head, channel) and starts fetching the partial outputs of the first 32
     // splits at once; meanwhile wave 0 fetches the (M, L) pairs, lane (s8, head) taking splits
     // s8, s8 + 8, ..., and turns them into one weight per split and head in LDS (the regions are
@@ -971,12 +1163,12 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     float* const tM = reinterpret_cast<float*>(lds);                  // [nsplit][8] maxima
     float* const tL = tM + P.nsplit * kMaxGroupHeads;                  // [nsplit][8] sums
     float* const sW = tL + P.nsplit * kMaxGroupHeads;                  // [8][nsp32] weights, zero past nsplit
-    const int64_t row00 = bi * P.h + hk * g;
+    const int64_t row00 = bi * n_h + hk * g;
     float v0[32], m8[8], l8[8];
     const int wl_hh = lane & 7, wl_s8 = lane >> 3;
     const int64_t wl_row = row00 + (wl_hh < g ? wl_hh : 0);
-    if (wave == 0) load_ml(m8, l8, P.ml_part, wl_row, hstride, 0, wl_s8, P.nsplit);     // ahead of the bulk loads
-    if (tid < g * kHeadDim) load_partials(v0, P.o_part, static_cast<uint32_t>((row00 + (tid >> 7)) * kHeadDim + (tid & 127)),
+    if (wave == 0) load_ml(m8, l8, ml_part, wl_row, hstride, 0, wl_s8, P.nsplit);     // ahead of the bulk loads
+    if (tid < g * kHeadDim) load_partials(v0, o_part, static_cast<uint32_t>((row00 + (tid >> 7)) * kHeadDim + (tid & 127)),
                                           hstride * kHeadDim, 0, P.nsplit);
     PROF(12);
     if (wave == 0) {
@@ -984,7 +1176,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         const bool live = hh < g;
         float M = -INFINITY;
         for (int sb = 0; sb < P.nsplit; sb += 64) {      // eight splits per lane and round
-            if (sb > 0) load_ml(m8, l8, P.ml_part, wl_row, hstride, sb, s8, P.nsplit);
+            if (sb > 0) load_ml(m8, l8, ml_part, wl_row, hstride, sb, s8, P.nsplit);
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const int sp = sb + s8 + 8 * k;
@@ -1022,7 +1214,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         float O = 0.0f;
         for (int s0 = 0; s0 < P.nsplit; s0 += 32) {
             if (idx != tid || s0 != 0) {
-                load_partials(v0, P.o_part, static_cast<uint32_t>((row00 + hh) * kHeadDim + c), hstride * kHeadDim, s0,
+                load_partials(v0, o_part, static_cast<uint32_t>((row00 + hh) * kHeadDim + c), hstride * kHeadDim, s0,
                               P.nsplit);
             }
 #pragma unroll
@@ -1036,16 +1228,19 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         }
         const float M = sHead[hh], L = sHead[kMaxGroupHeads + hh];
         const bool none = !(L > 0.0f);
-        P.out[bi * P.out_sb + hq * P.out_sh + c] = to_out<BF16>(none ? 0.0f : O / L);
-        if (c == 0 && P.lse) {
-            P.lse[row00 + hh] = none ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+        out[bi * out_sb + hq * out_sh + c] = to_out<BF16>(none ? 0.0f : O / L);
+        if (c == 0 && lse_out) {
+            lse_out[row00 + hh] = none ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
         }
     }
+    }   // nsplit > 1
+    // here: the workgroup that wrote the output of its (batch, kv-head)
+    if constexpr (APPEND) step_end<BITS, GS, BF16>(lds, bi, hk, step_len);
     PROF(7);
     PROF_FLUSH();
 }
 
-template <int BITS, int GS, bool BF16>
+template <int BITS, int GS, bool BF16, bool APPEND>
 hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
     constexpr int kLds = fwd_lds_bytes<BITS, GS>();
     // the dynamic-LDS limit is raised once per kernel and device (idempotent, so a race between
@@ -1054,19 +1249,22 @@ hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !configured[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16, APPEND>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return e;
         if (dev >= 0 && dev < 64) configured[dev] = true;
     }
-    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16>), dim3(P.nsplit * P.hk * P.b),
+    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16, APPEND>), dim3(P.nsplit * P.hk * P.b),
                        dim3(UnitCfg<BITS, GS>::NW * 64), kLds, stream, P);
     return hipGetLastError();
 }
 
 template <int BITS, int GS>
 hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
-    return P.bf16 ? launch_fwd_tt<BITS, GS, true>(P, stream) : launch_fwd_tt<BITS, GS, false>(P, stream);
+    if (P.lengths) {
+        return P.bf16 ? launch_fwd_tt<BITS, GS, true, true>(P, stream) : launch_fwd_tt<BITS, GS, false, true>(P, stream);
+    }
+    return P.bf16 ? launch_fwd_tt<BITS, GS, true, false>(P, stream) : launch_fwd_tt<BITS, GS, false, false>(P, stream);
 }
 
 }  // namespace

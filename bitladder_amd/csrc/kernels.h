@@ -23,6 +23,8 @@ struct QpackParams {
     int chunks_per_page;
 };
 
+// (The decode kernel fetches k_res ... vres_sh and o_part ... h as two 64-byte blocks: keep each group
+// contiguous and in this order; static_asserts in decode.hip check it.)
 struct FwdParams {
     const uint16_t* q;
     int64_t q_sb, q_sh;
@@ -51,6 +53,16 @@ struct FwdParams {
     const int* block_table;     // paged cache, as in QpackParams
     int64_t bt_stride;
     int chunks_per_page;
+    // Decode step with append (lengths != nullptr): sequence i holds lengths[i] tokens, the last
+    // lengths[i] % 128 of them in the fp16 window; its new token (k_new, v_new) is attended as the
+    // window's next row, stored there, and a window that becomes full is packed behind the prefix.
+    // seqlens / reslens / seqlen / reslen are not used then.
+    int* lengths;               // [b], advanced by one by the last workgroup of each sequence
+    int* step_tickets;          // [b] arrival counters, zero between calls
+    const uint16_t* k_new;
+    const uint16_t* v_new;
+    int64_t knew_sb, knew_sh, vnew_sb, vnew_sh;
+    int capacity;               // packed tokens a sequence can hold
 };
 
 hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);

@@ -168,15 +168,16 @@ class DecodePlan:
     Built by `plan_fwd_kvcache_int`; the tensors it was built from must stay alive and in place.
     """
 
-    def __init__(self, args: "_lib.FwdArgs", out: torch.Tensor, lse: Optional[torch.Tensor],
+    def __init__(self, args, out: torch.Tensor, lse: Optional[torch.Tensor],
                  keep: tuple, device: torch.device):
-        self.args = args
+        self.args = args            # FwdArgs, or FwdAppendArgs for a decode step with append
         self.out = out
         self.lse = lse
         self._keep = keep
         self.device = device
-        self.num_splits = args.num_splits
-        self._fn = _lib.lib().bitdecode_fwd
+        step = isinstance(args, _lib.FwdAppendArgs)
+        self.num_splits = args.fwd.num_splits if step else args.num_splits
+        self._fn = _lib.lib().bitdecode_fwd_append if step else _lib.lib().bitdecode_fwd
         self._ref = ctypes.byref(args)
 
     def run(self, stream: Optional[int] = None) -> torch.Tensor:
@@ -333,6 +334,88 @@ def fwd_kvcache_int(q: torch.Tensor,
     return_lse = kwargs.get("return_lse", False)
     plan = plan_fwd_kvcache_int(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale,
                                 quant_mode, group_size, num_bits, **kwargs)
+    with torch.cuda.device(plan.device):
+        plan.run()
+    return (plan.out, plan.lse) if return_lse else plan.out
+
+
+def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                                k_pack: torch.Tensor, k_params: torch.Tensor,
+                                v_pack: torch.Tensor, v_params: torch.Tensor,
+                                k_residual: torch.Tensor, v_residual: torch.Tensor,
+                                lengths: torch.Tensor, max_len: int,
+                                opt_block_table: Optional[torch.Tensor] = None,
+                                softmax_scale: float = 1.0,
+                                quant_mode: str = "k-channel",
+                                group_size: int = 128,
+                                num_bits: int = 4,
+                                *,
+                                num_splits: int = 0,
+                                out: Optional[torch.Tensor] = None,
+                                return_lse: bool = False) -> DecodePlan:
+    """Validates a decode step with append and returns its `DecodePlan`; see `fwd_kvcache_int_append`."""
+    if k_residual is None or v_residual is None or k_residual.dim() != 4 or k_residual.shape[1] < CHUNK:
+        raise RuntimeError(f"the residual window must hold at least {CHUNK} tokens")
+    max_len = int(max_len)
+    if max_len < 0:
+        raise RuntimeError("max_len must not be negative")
+    inner = plan_fwd_kvcache_int(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale, quant_mode,
+                                 group_size, num_bits, seqlen_k=0, k_residual=k_residual, v_residual=v_residual,
+                                 residual_len=CHUNK, num_splits=1, out=out, return_lse=return_lse)
+    device, b, h, h_k = inner.device, q.shape[0], q.shape[2], v_pack.shape[2]
+    for name, t in (("k_new", k_new), ("v_new", v_new)):
+        if t.dim() != 4 or tuple(t.shape) != (b, 1, h_k, 128):
+            raise RuntimeError(f"{name} must be [batch, 1, nheads_k, head_dim]")
+        if t.dtype != q.dtype or t.device != device:
+            raise RuntimeError(f"{name} must have the dtype and device of q")
+        if t.stride(3) != 1:
+            raise RuntimeError(f"{name} must have contiguous last dimension")
+    a = _lib.FwdAppendArgs()
+    a.fwd = inner.args
+    a.fwd.max_res_len = k_residual.shape[1]
+    a.lengths = _i32_dev(lengths, b, device, "lengths").data_ptr()
+    a.k_new, a.knew_stride_b, a.knew_stride_h = k_new.data_ptr(), k_new.stride(0), k_new.stride(2)
+    a.v_new, a.vnew_stride_b, a.vnew_stride_h = v_new.data_ptr(), v_new.stride(0), v_new.stride(2)
+    a.max_len = max_len
+    L = _lib.lib()
+    with torch.cuda.device(device):
+        ns = int(num_splits)
+        if ns == 0:
+            ns = L.bitdecode_num_splits(b, h_k, max_len // CHUNK * CHUNK, CHUNK, 0, num_bits, group_size)
+        a.fwd.num_splits = ns
+        nbytes = L.bitdecode_fwd_append_workspace_bytes(b, h, ns)
+        # zero-filled: the arrival counters must be 0 before the first call (every call leaves them at 0)
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        a.fwd.workspace, a.fwd.workspace_bytes = ws.data_ptr(), nbytes
+    keep = inner._keep + (k_new, v_new, lengths, ws)
+    return DecodePlan(a, inner.out, inner.lse, keep, device)
+
+
+def fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                           k_pack: torch.Tensor, k_params: torch.Tensor,
+                           v_pack: torch.Tensor, v_params: torch.Tensor,
+                           k_residual: torch.Tensor, v_residual: torch.Tensor,
+                           lengths: torch.Tensor, max_len: int,
+                           opt_block_table: Optional[torch.Tensor] = None,
+                           softmax_scale: float = 1.0,
+                           quant_mode: str = "k-channel",
+                           group_size: int = 128,
+                           num_bits: int = 4,
+                           **kwargs):
+    """One decode step in one launch (the "residual kernel" of the reference's figures,
+    imgs/overview.png and imgs/scheme.png; no code for it in the reference's main branch).
+
+    Sequence i holds `lengths[i]` tokens (int32 device tensor): whole blocks of 128 in the packed cache,
+    the remainder in rows 0.. of `k_residual / v_residual [b, >=128, h_k, 128]`.  The call attends
+    q [b, 1, h, 128] over all of them plus the new token `k_new / v_new [b, 1, h_k, 128]`, stores the
+    new token in the window, quantize-packs a window that reaches 128 tokens behind the prefix, and
+    advances `lengths` on the device.  `max_len` is a host upper bound of `lengths` before the step (it
+    sizes the grid; the capacity of the cache always works).  Keyword-only: num_splits, out, return_lse.
+    """
+    return_lse = kwargs.get("return_lse", False)
+    plan = plan_fwd_kvcache_int_append(q, k_new, v_new, k_pack, k_params, v_pack, v_params, k_residual, v_residual,
+                                       lengths, max_len, opt_block_table, softmax_scale, quant_mode, group_size,
+                                       num_bits, **kwargs)
     with torch.cuda.device(plan.device):
         plan.run()
     return (plan.out, plan.lse) if return_lse else plan.out

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define BITDECODE_ABI_VERSION 2
+#define BITDECODE_ABI_VERSION 3
 
 enum {
     BITDECODE_OK = 0,
@@ -108,6 +108,37 @@ typedef struct bitdecode_fwd_args {
 } bitdecode_fwd_args;
 
 int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
+
+/* One decode step in one launch: attend the new token together with everything held, append it, and
+ * quantize-pack the fp16 window when it fills.  This is the "residual kernel" the reference's figures
+ * describe (imgs/overview.png, imgs/scheme.png) and its kernel traits still name
+ * (csrc/bit_decode/src/include/kernel_traits.h:76,85: residual_block_size); the reference's main
+ * branch ships no code for it.  Sequence i holds lengths[i] tokens before the call: the first
+ * lengths[i] / 128 * 128 in the packed cache, the rest in rows 0.. of its window.  The call
+ *   - attends q over [packed prefix || window || new token],
+ *   - stores the new token in the window's next row,
+ *   - if that makes 128 rows, packs them into the cache behind the prefix (they were attended in
+ *     fp16 in this call and are read as codes from the next one on),
+ *   - sets lengths[i] += 1.
+ * A sequence whose window fills while its cache has no room for another 128 tokens is attended but
+ * left unchanged (its length does not advance).  Lengths stay on the device, so a captured HIP graph of
+ * this call can be replayed step after step with no host work.
+ * In `fwd`: seqlen_k, seqlens_k, res_len, res_lens and max_seqlen_k are ignored; k_res / v_res are the
+ * window (written), max_res_len its capacity in tokens (at least 128); the packed cache is written;
+ * workspace must hold bitdecode_fwd_append_workspace_bytes(...) bytes, required for any split count,
+ * zero before the first call. */
+typedef struct bitdecode_fwd_append_args {
+    bitdecode_fwd_args fwd;
+    int32_t* lengths;          /* device int32[b], read and advanced                        */
+    const void* k_new;         /* [b, 1, h_k, 128] element type of q, last dim contiguous   */
+    const void* v_new;
+    int64_t knew_stride_b, knew_stride_h;
+    int64_t vnew_stride_b, vnew_stride_h;
+    int32_t max_len;           /* host upper bound of lengths before the step (sizes the grid) */
+} bitdecode_fwd_append_args;
+
+int bitdecode_fwd_append(const bitdecode_fwd_append_args* args, void* stream);
+size_t bitdecode_fwd_append_workspace_bytes(int32_t b, int32_t h, int32_t num_splits);
 
 /* Split count the library would choose for this problem (host function, no GPU work);
  * replaces num_splits_heuristic (csrc/bit_decode/decode_api.cpp:234-268), retuned for 256 CUs.

@@ -20,6 +20,12 @@ def _pool(num_pages, page, h_k, bits, gs, device):
     return H.alloc_cache(num_pages, page, h_k, bits, gs, device, fill=0x5A5A)
 
 
+def _where(got, want):
+    """Which (sequence, head) rows differ, and by how much: for the message of a failed comparison."""
+    d = (got.float() - want.float()).abs().amax(dim=(1, 3))
+    return [(int(i), int(j), float(d[i, j])) for i, j in torch.nonzero(d)]
+
+
 def _region_bytes(t, regions):
     """Flat bytes of a cache tensor, one row per (batch-or-page, kv-head) region."""
     return t.contiguous().view(torch.uint8).reshape(regions, -1)
@@ -62,7 +68,7 @@ def test_paged_pack_and_decode_equal_contiguous(device, bits, gs, page):
                                max_seqlen_k=S, **kw)
         got = fwd_kvcache_int(qd, *pool, table, SCALE, "k-channel", gs, bits, num_splits=ns, seqlens_k=seqlens,
                               max_seqlen_k=S, **kw)
-        assert torch.equal(got, want), ns
+        assert torch.equal(got, want), (ns, _where(got, want))
     # and the paged result is right, not merely equal
     qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs)
     k_hat, v_hat = O.dequantize_ref(qkv)

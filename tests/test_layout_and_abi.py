@@ -110,7 +110,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_mirrors_match_header_field_order():
     header = open(os.path.join(ROOT, "include", "bitdecode.h")).read()
-    for cname, cls in (("bitdecode_qpack_args", _lib.QpackArgs), ("bitdecode_fwd_args", _lib.FwdArgs)):
+    for cname, cls in (("bitdecode_qpack_args", _lib.QpackArgs), ("bitdecode_fwd_args", _lib.FwdArgs),
+                       ("bitdecode_fwd_append_args", _lib.FwdAppendArgs)):
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cname, cname), header, re.S).group(1)
         body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
         names = []
