@@ -351,10 +351,19 @@ template <int BITS, int GS>
 __device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int bi, int hk, int u) {
     using C = UnitCfg<BITS, GS>;
     const int uic = u % C::UPC;
-    // region and chunk inside it (a paged cache looks the page up in the block table: a scalar load)
-    const ChunkPlace place = chunk_place(P.block_table, P.bt_stride, P.chunks_per_page, bi, hk, P.hk, u / C::UPC);
-    const int64_t bh = place.region;
-    const int ci = place.chunk;
+    // region and chunk inside it, as layout.h::chunk_place; a paged cache looks the page up in the block
+    // table with a scalar load written out here: a load the compiler tracks would be a vector load, and its
+    // wait would also drain the direct-to-LDS loads in flight
+    int ci = u / C::UPC;
+    int64_t bh = static_cast<int64_t>(bi) * P.hk + hk;
+    if (P.block_table) {
+        const int slot = ci / P.chunks_per_page;
+        int page;
+        asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                     : "=s"(page) : "s"(P.block_table + bi * P.bt_stride + slot) : "memory");
+        bh = static_cast<int64_t>(page) * P.hk + hk;
+        ci -= slot * P.chunks_per_page;
+    }
     UnitAddr<BITS, GS> A;      // wave-uniform: everything here lives in SGPRs
     A.kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
     A.vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
