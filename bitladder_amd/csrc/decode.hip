@@ -278,6 +278,14 @@ __device__ __forceinline__ void dma_row_first_lanes(const uint8_t* base, uint32_
 
 // s_waitcnt vmcnt(n): at most n of this wave's loads still in flight.  The compiler does not
 // track the asm loads above, so the waits are explicit; the memory clobber keeps LDS reads below.
+// All of this wave's LDS reads have returned their data.  A direct-to-LDS load may be given an LDS
+// location only after that: a read that has merely been issued can still be overtaken by the load's
+// write when the data comes from a near cache and the LDS queue is long (seen as rare wrong results
+// with twelve waves of the 4-bit, group-32 kernel and L2-resident caches).
+__device__ __forceinline__ void wait_lds_reads() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -337,7 +345,7 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 // The loads of a unit, in the order they are consumed: K side (K parameters, four K code rows), then
 // V side (V parameters, four V code rows).  A wave issues both sides of its first unit at once.
 // After that the next unit's K side is issued as soon as the current unit's last QK^T has read the
-// K rows, into the same rows and into the other K-parameter slot, and its V side as soon as the last
+// K rows (and the data of those reads has come back: wait_lds_reads), into the same rows and into the other K-parameter slot, and its V side as soon as the last
 // PV has read the V rows and V parameters: the next unit is on its way while the current one is
 // being computed, without a second code buffer.
 template <int BITS, int GS>
@@ -516,7 +524,10 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
             for (int r = 0; r < 4; ++r) t[4 * tt + r] = acc[r] + partner(acc[r]);   // hi + lo
         }
         // every K row and this unit's K parameters have been read: the next unit's K side may land
-        if (HAS_NEXT && step == kLast) issue_kside<BITS, GS>(next, lane * 16, region_lds, kslot ^ 1);
+        if (HAS_NEXT && step == kLast) {
+            wait_lds_reads();
+            issue_kside<BITS, GS>(next, lane * 16, region_lds, kslot ^ 1);
+        }
         PHASE(10 + 3 * step);
 
         softmax_step<4 * TPS, NCG>(t, P.scale_log2, st);
@@ -571,7 +582,10 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
         }
     }
     // every V row and the V parameters have been read: the next unit's V side may land
-    if (HAS_NEXT) issue_vside<BITS, GS>(next, lane * 16, region_lds);
+    if (HAS_NEXT) {
+        wait_lds_reads();
+        issue_vside<BITS, GS>(next, lane * 16, region_lds);
+    }
     PHASE(15);
 }
 

@@ -260,3 +260,24 @@ def test_qpack_ranges_from_subnormal_to_max(device, bits, dtype):
     cache = _pack_gpu(k, v, bits, gs, dtype, device, S)
     torch.cuda.synchronize()
     H.assert_cache_equals_oracle(H.cache_to_numpy(*cache), want)
+
+
+@pytest.mark.parametrize("bits,gs,S,ns", [(4, 32, 4096, 1), (4, 32, 8192, 2), (4, 128, 8192, 1), (2, 64, 16384, 1)])
+def test_waves_with_many_units_on_cache_resident_data_are_deterministic(device, bits, gs, S, ns):
+    """Each wave streams three or more units through its LDS region, and the cache is small enough to stay in
+    L2 while the call is repeated: the direct-to-LDS loads of the next unit then come back fast, and must
+    still not overtake the LDS reads of the current one (the kernel waits for those reads before it issues
+    the loads).  Every repetition must give the same bits, and the right ones."""
+    from bitladder_amd import fwd_kvcache_int, kvcache_pack_int
+    b, h, h_k = 1, 8, 2
+    q, k, v = O.make_inputs(b, h, h_k, S, 0, seed=61)
+    qd, kd, vd = H.to_dev(q, "fp16", device), H.to_dev(k, "fp16", device), H.to_dev(v, "fp16", device)
+    cache = H.alloc_cache(b, S, h_k, bits, gs, device)
+    kvcache_pack_int(kd, cache[0], cache[1], vd, cache[2], cache[3], None, None, S, "k-channel", gs, bits)
+    outs = [fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns) for _ in range(200)]
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, outs[0]) for o in outs[1:])
+    qkv = O.quantize_kv_ref(k, v, bits, gs)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    ref, _ = O.attend_ref(q, k_hat, v_hat, SCALE)
+    assert np.abs(outs[0].float().cpu().numpy() - ref).max() < 2e-3
