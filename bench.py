@@ -28,6 +28,10 @@ HBM_PEAK_GBS = 8000.0
 # counter is in units of 2 KiB and the write counter in KiB.
 MEASURED_TRAFFIC_BYTES = {
     "llama3-8b-gqa-32k-4bit-g128": int(18089.2 * 2048 + 592.25 * 1024),
+    # the other workloads, same method (profiles/fwd_splitkv_hbm_traffic_all_workloads.md)
+    "llama2-7b-mha-4k-4bit-g128": int(9955.41 * 2048 + 161.0 * 1024),
+    "llama3-8b-gqa-128k-2bit-g64": int(41731.14 * 2048 + 592.25 * 1024),
+    "llama3-70b-gqa-64k-2bit-g128-b8": int(150316.26 * 2048 + 1290.0 * 1024),
 }
 
 WORKLOADS = {
