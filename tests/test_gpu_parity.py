@@ -233,6 +233,10 @@ def test_decode_random_shapes(device, seed):
     err = np.abs(out.float().cpu().numpy() - want).max()
     assert err < tol, (bits, gs, dtype, b, h, h_k, S, R, ns, err)
     np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=3e-3, rtol=1e-4)
+    # and the same bits every time, also once the cache has become L2-resident
+    for _ in range(20):
+        again, _ = fwd_kvcache_int(H.to_dev(q, dtype, device), *cache, None, scale, "k-channel", gs, bits, **kw)
+        assert torch.equal(again, out)
 
 
 @pytest.mark.parametrize("bits", [2, 4])
