@@ -43,6 +43,8 @@ struct Api {
     size_t (*workspace_bytes)(int32_t, int32_t, int32_t);
     int (*qpack)(const bitdecode_qpack_args*, void*);
     int (*fwd)(const bitdecode_fwd_args*, void*);
+    int (*fwd_append)(const bitdecode_fwd_append_args*, void*);
+    size_t (*fwd_append_workspace_bytes)(int32_t, int32_t, int32_t);
 };
 typedef void (*quantize_fn)(const float*, const float*, int, int, int, int, int, int, int, uint8_t*, float*, float*,
                             uint8_t*, float*, float*);
@@ -239,6 +241,145 @@ bool run_case(const Api& api, quantize_fn quantize, attend_fn attend, round_fn r
     return ok;
 }
 
+// A decode loop on the one-launch entry point: every sequence starts with `start` tokens (whole 128-token
+// blocks packed with bitdecode_qpack, the rest copied into its fp16 window) and takes `steps` calls of
+// bitdecode_fwd_append, each with a new token and a new query; lengths stay on the device.  Checked at the
+// end: the length counters, and the last call's output against the C restatement on the token history
+// (blocks that were packed -- by the pack call or inside a step -- read as codes, the rest as fp16).
+bool run_step_case(const Api& api, quantize_fn quantize, attend_fn attend, round_fn round16, int b, int h, int hk,
+                   int start, int steps, int bits, int gs) {
+    const int d = 128, pn = 16 / bits, n = start + steps;
+    const int cap = (n + 127) / 128 * 128;
+    std::mt19937 rng(7);
+    std::normal_distribution<float> gauss(0.f, 1.f);
+    const size_t row = static_cast<size_t>(hk) * d;
+    std::vector<float> q(static_cast<size_t>(steps) * b * h * d), k(static_cast<size_t>(b) * n * row), v(k.size());
+    for (auto& x : q) x = round16(gauss(rng));
+    for (auto& x : k) x = round16(gauss(rng));
+    for (auto& x : v) x = round16(gauss(rng));
+    std::vector<uint16_t> qh(q.size()), kh(k.size()), vh(v.size());
+    for (size_t i = 0; i < q.size(); ++i) qh[i] = f32_to_f16_bits(q[i]);
+    for (size_t i = 0; i < k.size(); ++i) kh[i] = f32_to_f16_bits(k[i]);
+    for (size_t i = 0; i < v.size(); ++i) vh[i] = f32_to_f16_bits(v[i]);
+    uint16_t *dq = to_device(qh), *dk = to_device(kh), *dv = to_device(vh);
+
+    const size_t pack_bytes = static_cast<size_t>(b) * cap / pn * row * 2;
+    const size_t param_bytes = static_cast<size_t>(b) * cap / gs * row * 4;
+    const size_t win_bytes = static_cast<size_t>(b) * 128 * row * 2;
+    void *k_pack, *k_params, *v_pack, *v_params, *out, *k_win, *v_win, *lengths, *workspace;
+    HIP_OK(hipMalloc(&k_pack, pack_bytes));
+    HIP_OK(hipMalloc(&v_pack, pack_bytes));
+    HIP_OK(hipMalloc(&k_params, param_bytes));
+    HIP_OK(hipMalloc(&v_params, param_bytes));
+    HIP_OK(hipMalloc(&out, static_cast<size_t>(b) * h * d * 2));
+    HIP_OK(hipMalloc(&k_win, win_bytes));
+    HIP_OK(hipMalloc(&v_win, win_bytes));
+    HIP_OK(hipMalloc(&lengths, b * sizeof(int32_t)));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+
+    // prefill: whole blocks packed, the remainder into the window
+    const int packed0 = start / 128 * 128, r0 = start - packed0;
+    if (packed0) {
+        bitdecode_qpack_args pa;
+        std::memset(&pa, 0, sizeof pa);
+        pa.k = dk; pa.v = dv;
+        pa.k_stride_b = pa.v_stride_b = static_cast<int64_t>(n) * row;
+        pa.k_stride_t = pa.v_stride_t = static_cast<int64_t>(row);
+        pa.k_stride_h = pa.v_stride_h = d;
+        pa.k_pack = k_pack; pa.k_params = k_params; pa.v_pack = v_pack; pa.v_params = v_params;
+        pa.b = b; pa.n_tokens = packed0; pa.h_k = hk; pa.d = d;
+        pa.cache_tokens = cap;
+        pa.bits = bits; pa.group_size = gs; pa.dtype = BITDECODE_FP16;
+        if (int rc = api.qpack(&pa, stream)) {
+            std::fprintf(stderr, "bitdecode_qpack failed (%d): %s\n", rc, api.last_error());
+            return false;
+        }
+    }
+    for (int bi = 0; bi < b && r0; ++bi) {
+        const size_t src = (static_cast<size_t>(bi) * n + packed0) * row, dst = static_cast<size_t>(bi) * 128 * row;
+        HIP_OK(hipMemcpyAsync(static_cast<uint16_t*>(k_win) + dst, dk + src, r0 * row * 2, hipMemcpyDeviceToDevice, stream));
+        HIP_OK(hipMemcpyAsync(static_cast<uint16_t*>(v_win) + dst, dv + src, r0 * row * 2, hipMemcpyDeviceToDevice, stream));
+    }
+    std::vector<int32_t> len0(b, start);
+    HIP_OK(hipMemcpyAsync(lengths, len0.data(), b * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+
+    const float scale = 1.f / std::sqrt(static_cast<float>(d));
+    bitdecode_fwd_append_args sa;
+    std::memset(&sa, 0, sizeof sa);
+    bitdecode_fwd_args& fa = sa.fwd;
+    fa.q_stride_b = static_cast<int64_t>(h) * d; fa.q_stride_h = d;
+    fa.k_pack = k_pack; fa.k_params = k_params; fa.v_pack = v_pack; fa.v_params = v_params;
+    fa.cache_tokens = cap;
+    fa.k_res = k_win; fa.v_res = v_win;
+    fa.kres_stride_b = fa.vres_stride_b = 128 * static_cast<int64_t>(row);
+    fa.kres_stride_t = fa.vres_stride_t = static_cast<int64_t>(row);
+    fa.kres_stride_h = fa.vres_stride_h = d;
+    fa.max_res_len = 128;                        // capacity of the window
+    fa.out = out; fa.out_stride_b = static_cast<int64_t>(h) * d; fa.out_stride_h = d;
+    fa.b = b; fa.h = h; fa.h_k = hk; fa.d = d;
+    fa.bits = bits; fa.group_size = gs; fa.dtype = BITDECODE_FP16;
+    fa.softmax_scale = scale;
+    fa.num_splits = api.num_splits(b, hk, cap, 128, 0, bits, gs);   // one grid for every step
+    const size_t ws = api.fwd_append_workspace_bytes(b, h, fa.num_splits);
+    HIP_OK(hipMalloc(&workspace, ws));
+    HIP_OK(hipMemsetAsync(workspace, 0, ws, stream));
+    fa.workspace = workspace;
+    fa.workspace_bytes = ws;
+    sa.lengths = static_cast<int32_t*>(lengths);
+    sa.knew_stride_b = sa.vnew_stride_b = static_cast<int64_t>(n) * row;
+    sa.knew_stride_h = sa.vnew_stride_h = d;
+    sa.max_len = cap + 127;
+    for (int s = 0; s < steps; ++s) {
+        fa.q = dq + static_cast<size_t>(s) * b * h * d;
+        sa.k_new = dk + static_cast<size_t>(start + s) * row;     // token start + s of every sequence
+        sa.v_new = dv + static_cast<size_t>(start + s) * row;
+        if (int rc = api.fwd_append(&sa, stream)) {
+            std::fprintf(stderr, "bitdecode_fwd_append failed (%d): %s\n", rc, api.last_error());
+            return false;
+        }
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<uint16_t> oh(static_cast<size_t>(b) * h * d);
+    std::vector<int32_t> len1(b);
+    HIP_OK(hipMemcpy(oh.data(), out, oh.size() * 2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(len1.data(), lengths, b * sizeof(int32_t), hipMemcpyDeviceToHost));
+    bool ok = true;
+    for (int bi = 0; bi < b; ++bi) ok = ok && len1[bi] == n;
+
+    // the last call saw n - 1 tokens plus its new one: blocks below `packed` as codes, the rest fp16
+    const int packed = (n - 1) / 128 * 128, R = n - packed;
+    std::vector<float> kp(static_cast<size_t>(b) * packed * row), vp(kp.size()), kr(static_cast<size_t>(b) * R * row), vr(kr.size());
+    for (int bi = 0; bi < b; ++bi) {
+        if (packed) {
+            std::memcpy(&kp[static_cast<size_t>(bi) * packed * row], &k[static_cast<size_t>(bi) * n * row], packed * row * 4);
+            std::memcpy(&vp[static_cast<size_t>(bi) * packed * row], &v[static_cast<size_t>(bi) * n * row], packed * row * 4);
+        }
+        std::memcpy(&kr[static_cast<size_t>(bi) * R * row], &k[(static_cast<size_t>(bi) * n + packed) * row], R * row * 4);
+        std::memcpy(&vr[static_cast<size_t>(bi) * R * row], &v[(static_cast<size_t>(bi) * n + packed) * row], R * row * 4);
+    }
+    std::vector<uint8_t> kc(kp.size() + 1), vc(kp.size() + 1);
+    std::vector<float> ks(kp.size() / gs + 1), kz(ks.size()), vs(ks.size()), vz(ks.size());
+    if (packed)
+        quantize(kp.data(), vp.data(), b, packed, hk, d, bits, gs, 0, kc.data(), ks.data(), kz.data(), vc.data(), vs.data(),
+                 vz.data());
+    std::vector<float> want(oh.size()), lse(static_cast<size_t>(b) * h);
+    attend(&q[static_cast<size_t>(steps - 1) * b * h * d], kc.data(), ks.data(), kz.data(), vc.data(), vs.data(), vz.data(),
+           kr.data(), vr.data(), nullptr, nullptr, b, h, hk, d, packed, R, gs, scale, want.data(), lse.data());
+    double max_err = 0;
+    for (size_t i = 0; i < oh.size(); ++i) max_err = std::fmax(max_err, std::fabs(f16_bits_to_f32(oh[i]) - want[i]));
+    ok = ok && max_err < 2e-3;
+    std::printf("decode loop, b %d heads %d/%d, %d tokens + %d steps of bitdecode_fwd_append, %d-bit g%d, %d splits: "
+                "lengths %d, last step max|out - dequant-attend| %.2e -> %s\n",
+                b, h, hk, start, steps, bits, gs, fa.num_splits, len1[0], max_err, ok ? "pass" : "FAIL");
+    std::fflush(stdout);
+    for (void* p : {static_cast<void*>(dq), static_cast<void*>(dk), static_cast<void*>(dv), k_pack, k_params, v_pack,
+                    v_params, out, k_win, v_win, lengths, workspace})
+        HIP_OK(hipFree(p));
+    HIP_OK(hipStreamDestroy(stream));
+    return ok;
+}
+
 }  // namespace
 
 extern "C" int packdecode_driver_run(const char* lib_path, const char* oracle_path) {
@@ -255,6 +396,8 @@ extern "C" int packdecode_driver_run(const char* lib_path, const char* oracle_pa
     api.workspace_bytes = sym<decltype(api.workspace_bytes)>(lib, "bitdecode_fwd_workspace_bytes");
     api.qpack = sym<decltype(api.qpack)>(lib, "bitdecode_qpack");
     api.fwd = sym<decltype(api.fwd)>(lib, "bitdecode_fwd");
+    api.fwd_append = sym<decltype(api.fwd_append)>(lib, "bitdecode_fwd_append");
+    api.fwd_append_workspace_bytes = sym<decltype(api.fwd_append_workspace_bytes)>(lib, "bitdecode_fwd_append_workspace_bytes");
     if (api.abi_version() != BITDECODE_ABI_VERSION) {
         std::fprintf(stderr, "ABI version %d, header says %d\n", api.abi_version(), BITDECODE_ABI_VERSION);
         return 2;
@@ -272,6 +415,9 @@ extern "C" int packdecode_driver_run(const char* lib_path, const char* oracle_pa
     };
     int failed = 0;
     for (const Case& c : cases) failed += !run_case(api, quantize, attend, round16, c);
+    // decode loops across a window that fills (once, and twice with an empty start)
+    failed += !run_step_case(api, quantize, attend, round16, 2, 32, 8, 1024 + 100, 40, 4, 128);
+    failed += !run_step_case(api, quantize, attend, round16, 1, 16, 2, 0, 260, 2, 64);
     std::printf("%d case(s) failed\n", failed);
     std::fflush(stdout);
     return failed ? 1 : 0;
