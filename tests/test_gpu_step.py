@@ -274,3 +274,40 @@ def test_step_packs_exactly_what_the_pack_kernel_packs(device, bits, gs, dtype):
     for g_, w_ in zip(got, want):
         assert torch.equal(g_, w_)
 
+
+
+def test_step_on_a_ragged_batch_of_sixteen(device):
+    """The batch shape of the reference's batched driver (csrc/bit_decode/src/test_batch_packdecode.cu: 16
+    sequences, 32 query / 8 kv heads) with ragged lengths: 128 workgroup groups share the XCD-aware block
+    mapping, every sequence has eight ticket holders, and windows fill at different steps."""
+    from bitladder_amd import BitKVCache
+    b, h, h_k, steps, capacity = 16, 32, 8, 135, 2048 + 256
+    rng = np.random.default_rng(4)
+    lengths = [int(x) for x in rng.integers(1024, 2049, b)]
+    qs, k, v, qd, kd, vd = _inputs(b, h, h_k, 2048 + steps, "fp16", device, 77)
+    cache = BitKVCache(b, h_k, capacity, device=device)
+    manual = _Manual(b, h_k, capacity, 4, 128, torch.float16, device)
+    cache.prefill(kd[:, :2048], vd[:, :2048], lengths)
+    manual.prefill(kd[:, :2048], vd[:, :2048], lengths)
+    for s in range(steps):
+        t = 2048 + s
+        out = cache.step(qd[s], kd[:, t:t + 1], vd[:, t:t + 1], SCALE, num_splits=2)
+        want = manual.step(qd[s], kd[:, t:t + 1], vd[:, t:t + 1], 2)
+        assert torch.equal(out, want), s
+    assert cache.total.tolist() == manual.total == [x + steps for x in lengths]
+    for i in range(b):       # blocks packed during the loop (prefill leaves padding blocks behind short sequences)
+        lo, hi = lengths[i] // 128 * 128, (lengths[i] + steps) // 128 * 128
+        assert torch.equal(cache.v_pack[i, lo:hi], manual.cache[2][i, lo:hi])
+        assert torch.equal(cache.k_pack[i, lo // 4:hi // 4], manual.cache[0][i, lo // 4:hi // 4])
+        assert torch.equal(cache.k_params[i, lo // 128:hi // 128], manual.cache[1][i, lo // 128:hi // 128])
+        assert torch.equal(cache.v_params[i, :, :, lo:hi], manual.cache[3][i, :, :, lo:hi])
+    # the fused path against the oracle on the full history of one sequence
+    i = int(np.argmax(lengths))
+    L = lengths[i] + steps
+    hist_k = np.concatenate([k[i, :lengths[i]], k[i, 2048:2048 + steps]], 0)
+    hist_v = np.concatenate([v[i, :lengths[i]], v[i, 2048:2048 + steps]], 0)
+    P = (L - 1) // 128 * 128
+    qkv = O.quantize_kv_ref(hist_k[None, :P], hist_v[None, :P], 4, 128)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    ref, _ = O.attend_ref(qs[steps - 1][i:i + 1], k_hat, v_hat, SCALE, hist_k[None, P:], hist_v[None, P:])
+    assert np.abs(out[i:i + 1].float().cpu().numpy() - ref).max() < 2e-3
