@@ -3,8 +3,9 @@
 
 A step is one decode-attention call (split-KV kernel + combine) over one batch of synthetic
 input.  Workload = Llama-3-8B-shape GQA decode: batch 1, 32 q heads / 8 kv heads, head_dim 128,
-32768 packed tokens at 4 bits (group 128) plus a 128-token fp16 residual window.
-Prints ONE JSON line; see --help for the side measurements it carries.
+32768 packed tokens at 4 bits (group 128) plus a 128-token fp16 residual window (--workload selects the
+other shapes, among them a ragged batch of 16).  Prints ONE JSON line; see --help for the side
+measurements it carries.
 """
 from __future__ import annotations
 
@@ -40,7 +41,21 @@ WORKLOADS = {
     "llama2-7b-mha-4k-4bit-g128": (1, 32, 32, 4096, 128, 4, 128, torch.float16),
     "llama3-8b-gqa-128k-2bit-g64": (1, 32, 8, 131072, 128, 2, 64, torch.float16),
     "llama3-70b-gqa-64k-2bit-g128-b8": (8, 64, 8, 65536, 128, 2, 128, torch.bfloat16),
+    # ragged batch: 16 sequences of seeded lengths in [1024, 8192]; S is the cache capacity, R the window
+    # capacity.  Whole 128-token blocks of a sequence are packed; the remainder (< 128) plus the 128 newest
+    # tokens stay in the fp16 window (128-255 tokens), as in a decode loop just before the next block is packed.
+    "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": (16, 32, 8, 8192, 256, 4, 128, torch.float16),
 }
+RAGGED = {"llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": (1024, 8192)}
+
+
+def ragged_lengths(name, b):
+    """(packed tokens, window tokens) per sequence of a ragged workload, from a fixed seed."""
+    lo, hi = RAGGED[name]
+    g = torch.Generator().manual_seed(0)
+    total = torch.randint(lo, hi + 1, (b,), generator=g)
+    packed = (total - 128).clamp(min=0) // 128 * 128         # the newest 128 tokens are still in the window
+    return packed.to(torch.int32), (total - packed).to(torch.int32)
 
 
 def make_inputs(b, h, h_k, n_tokens, seed, dtype):
@@ -171,7 +186,15 @@ def main():
     torch.cuda.set_device(dev)
     b, h, h_k, S, R, bits, gs, dtype = WORKLOADS[args.workload]
     scale = 1.0 / math.sqrt(128)
-    total_bytes, packed_bytes = algorithmic_bytes(b, h, h_k, S, R, bits, gs)
+    ragged = args.workload in RAGGED
+    if ragged:
+        packed_len, win_len = ragged_lengths(args.workload, b)
+        per_tok = h_k * 128 * 2
+        packed_bytes = int(packed_len.sum().item() * per_tok * (bits / 8 + 4 / gs))
+        total_bytes = packed_bytes + int(win_len.sum().item()) * per_tok * 2 + 2 * b * h * 128 * 2
+        packed_dev, win_dev = packed_len.to(dev), win_len.to(dev)
+    else:
+        total_bytes, packed_bytes = algorithmic_bytes(b, h, h_k, S, R, bits, gs)
 
     # enough distinct caches that consecutive steps cannot be served from the Infinity Cache
     nbuf = 1 if args.no_rotate else max(2, math.ceil(320e6 / total_bytes))
@@ -186,9 +209,21 @@ def main():
         cache = alloc_cache(b, S, h_k, bits, gs, dev)
         kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S,
                          "k-channel", gs, bits)
-        kres, vres = kd[:, S:].contiguous(), vd[:, S:].contiguous()
-        plan = plan_fwd_kvcache_int(q.to(dev), *cache, None, scale, "k-channel", gs, bits,
-                                    k_residual=kres, v_residual=vres, num_splits=args.num_splits)
+        if ragged:
+            # window of sequence j: its tokens behind the packed prefix
+            kres = torch.zeros((b, R, h_k, 128), dtype=dtype, device=dev)
+            vres = torch.zeros_like(kres)
+            for j in range(b):
+                p0, r0 = int(packed_len[j]), int(win_len[j])
+                kres[j, :r0], vres[j, :r0] = kd[j, p0:p0 + r0], vd[j, p0:p0 + r0]
+            plan = plan_fwd_kvcache_int(q.to(dev), *cache, None, scale, "k-channel", gs, bits,
+                                        seqlens_k=packed_dev, max_seqlen_k=int(packed_len.max()),
+                                        k_residual=kres, v_residual=vres, residual_len=win_dev,
+                                        max_residual_len=int(win_len.max()), num_splits=args.num_splits)
+        else:
+            kres, vres = kd[:, S:].contiguous(), vd[:, S:].contiguous()
+            plan = plan_fwd_kvcache_int(q.to(dev), *cache, None, scale, "k-channel", gs, bits,
+                                        k_residual=kres, v_residual=vres, num_splits=args.num_splits)
         plans.append(plan)
         keep.append((cache, kres, vres))
         if i < 2 and not args.no_qpack:
@@ -228,7 +263,8 @@ def main():
         "data": "synthetic: seeded N(0,1) q/k/v, 3 of 128 K channels per kv-head x10, packed by the library's own "
                 "quantize-pack kernel",
         "config": {"workload": args.workload, "batch": b, "q_heads": h, "kv_heads": h_k, "head_dim": 128,
-                   "packed_tokens": S, "residual_tokens": R, "bits": bits, "group_size": gs,
+                   "packed_tokens": packed_len.tolist() if ragged else S,
+                   "residual_tokens": win_len.tolist() if ragged else R, "bits": bits, "group_size": gs,
                    "num_splits": plans[0].num_splits, "kv_buffers_rotated": nbuf,
                    "launch": "hip-graph" if graphed else "eager"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -254,18 +290,23 @@ def main():
             j = i % len(srcs)
             kd, vd = srcs[j]
             c = keep[j][0]
-            kvcache_pack_int(kd[:, S - 128:S], c[0], c[1], vd[:, S - 128:S], c[2], c[3], None, None, 128,
-                             "k-channel", gs, bits, dst_offset=S - 128)
+            if ragged:      # every sequence's next block, at its own position
+                kvcache_pack_int(kd[:, S - 128:S], c[0], c[1], vd[:, S - 128:S], c[2], c[3], None, None, 128,
+                                 "k-channel", gs, bits, dst_offsets=packed_dev)
+            else:
+                kvcache_pack_int(kd[:, S - 128:S], c[0], c[1], vd[:, S - 128:S], c[2], c[3], None, None, 128,
+                                 "k-channel", gs, bits, dst_offset=S - 128)
 
         n_pack = max(10, args.steps // 4)
         _, ep, _ = time_steps(pack_all, n_pack, 3, not args.no_graph)
         _, ea, _ = time_steps(pack_block, args.steps, args.warmup, not args.no_graph)
         us_pack, us_app = ep / n_pack * 1e6, ea / args.steps * 1e6
         rd = b * h_k * S * 128 * 2 * 2
-        gbs = (rd + packed_bytes) / (us_pack * 1e-6) / 1e9
+        wr = int(b * h_k * S * 128 * 2 * (bits / 8 + 4 / gs))      # the whole capacity is packed
+        gbs = (rd + wr) / (us_pack * 1e-6) / 1e9
         result["qpack"] = {
             "kernel": "qpack_kernel", "bound": "hbm", "tokens": S, "us_per_call": round(us_pack, 3),
-            "bytes_read": rd, "bytes_written": packed_bytes, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+            "bytes_read": rd, "bytes_written": wr, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
             "append_128_tokens_us_per_call": round(us_app, 3)}
         srcs.clear()
@@ -279,7 +320,7 @@ def main():
         splans = []
         for i in range(n_slots):
             cache, kres, vres = keep[i % nbuf]
-            lengths = torch.full((b,), S + 64, dtype=torch.int32, device=dev)
+            lengths = ((packed_dev + 64) if ragged else torch.full((b,), S + 64, device=dev)).to(torch.int32)
             q_t = torch.randn((b, 1, h, 128), device=dev).to(dtype)
             kn = torch.randn((b, 1, h_k, 128), device=dev).to(dtype)
             splans.append(plan_fwd_kvcache_int_append(q_t, kn, kn.clone(), *cache, kres.clone(), vres.clone(), lengths,
@@ -300,18 +341,22 @@ def main():
         for i in range(nb16):
             q, k, v = make_inputs(b, h, h_k, S + R, seed=100 + i, dtype=dtype)
             kd, vd = k.to(dev), v.to(dev)
+            kw16 = dict(residual_len=packed_dev + win_dev, max_residual_len=S + R) if ragged else {}
             fplans.append((plan_fwd_kvcache_int(q.to(dev), *dummy, None, scale, "k-channel", gs, bits, seqlen_k=0,
-                                                k_residual=kd, v_residual=vd), q.to(dev), kd, vd))
+                                                k_residual=kd, v_residual=vd, **kw16), q.to(dev), kd, vd))
         torch.cuda.synchronize(dev)
         w16, e16, _ = time_steps(lambda i: fplans[i % nb16][0].run(), args.steps, args.warmup, not args.no_graph)
         us16 = e16 / args.steps * 1e6
-        fp16_bytes = b * h_k * (S + R) * 128 * 2 * 2 + 2 * b * h * 128 * 2
+        fp16_tokens = int((packed_len + win_len).sum()) if ragged else b * (S + R)
+        fp16_bytes = fp16_tokens * h_k * 128 * 2 * 2 + 2 * b * h * 128 * 2
 
         def sdpa(i):
             _, qd, kd, vd = fplans[i % nb16]
             torch.nn.functional.scaled_dot_product_attention(
                 qd.transpose(1, 2), kd.transpose(1, 2), vd.transpose(1, 2), scale=scale, enable_gqa=True)
         try:
+            if ragged:
+                raise RuntimeError("not run on a ragged batch (SDPA would attend the padding as well)")
             _, es, _ = time_steps(sdpa, max(10, args.steps // 4), 3, False)
             us_sdpa = es / max(10, args.steps // 4) * 1e6
         except Exception as e:  # noqa: BLE001
@@ -323,7 +368,9 @@ def main():
             "torch_sdpa_us_per_step": None if us_sdpa is None else round(us_sdpa, 3)}
         del fplans
 
-    if not args.no_cpu:
+    if not args.no_cpu and ragged:
+        print("[bench] the CPU baseline leg runs on the uniform workloads only", file=sys.stderr)
+    elif not args.no_cpu:
         out_cpu, t_cpu, reps = cpu_baseline(q0, k0, v0, S, R, bits, gs, scale)
         out_gpu = plans[0].run().float().cpu()
         torch.cuda.synchronize(dev)
