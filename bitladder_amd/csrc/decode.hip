@@ -246,9 +246,10 @@ struct UnitCfg {
 };
 
 // 16 bytes per lane from global memory straight into LDS: lane l reads base + OFFSET + 16*l and its
-// data lands at lds_base + OFFSET + 16*l (the instruction's immediate offset applies to both sides).  The base is wave-uniform and travels in SGPRs, the per-lane part is
-// one shared VGPR (lane16 = 16*lane), so the addresses of a whole unit cost no vector registers.
-// M0 carries the LDS byte address of the row.
+// data lands at lds_base + OFFSET + 16*l (the instruction's immediate offset applies to both sides).
+// The base is wave-uniform and travels in SGPRs, the per-lane part is one shared VGPR
+// (lane16 = 16*lane), so the addresses of a whole unit cost no vector registers.  M0 carries the
+// LDS byte address of the row.
 template <int OFFSET>
 __device__ __forceinline__ void dma_row(const uint8_t* base, uint32_t lane16, uint32_t lds_base) {
     static_assert(OFFSET >= 0 && OFFSET < 4096, "immediate offset field");
@@ -276,8 +277,6 @@ __device__ __forceinline__ void dma_row_first_lanes(const uint8_t* base, uint32_
                  : "memory", "m0", "scc");
 }
 
-// s_waitcnt vmcnt(n): at most n of this wave's loads still in flight.  The compiler does not
-// track the asm loads above, so the waits are explicit; the memory clobber keeps LDS reads below.
 // All of this wave's LDS reads have returned their data.  A direct-to-LDS load may be given an LDS
 // location only after that: a read that has merely been issued can still be overtaken by the load's
 // write when the data comes from a near cache and the LDS queue is long (seen as rare wrong results
@@ -286,6 +285,8 @@ __device__ __forceinline__ void wait_lds_reads() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 }
 
+// s_waitcnt vmcnt(n): at most n of this wave's loads still in flight.  The compiler does not
+// track the asm loads above, so the waits are explicit; the memory clobber keeps LDS reads below.
 template <int N>
 __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -345,9 +346,10 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 // The loads of a unit, in the order they are consumed: K side (K parameters, four K code rows), then
 // V side (V parameters, four V code rows).  A wave issues both sides of its first unit at once.
 // After that the next unit's K side is issued as soon as the current unit's last QK^T has read the
-// K rows (and the data of those reads has come back: wait_lds_reads), into the same rows and into the other K-parameter slot, and its V side as soon as the last
-// PV has read the V rows and V parameters: the next unit is on its way while the current one is
-// being computed, without a second code buffer.
+// K rows (and the data of those reads has come back: wait_lds_reads), into the same rows and into
+// the other K-parameter slot, and its V side as soon as the last PV has read the V rows and V
+// parameters: the next unit is on its way while the current one is being computed, without a
+// second code buffer.
 template <int BITS, int GS>
 struct UnitAddr {
     const uint8_t* kc;
@@ -667,8 +669,10 @@ __device__ __forceinline__ WindowSrc window_src(const FwdParams& P, int bi, int 
     // The decode step needs more parameter fields than the scalar registers hold next to the unit loop's
     // state: what the loop does not use is fetched from the kernarg segment only here.
     const kblock kb = karg_block<BLOCK_AT(k_res)>();      // k_res ... vres_sh
-    W.kr = BLOCK_PTR(const uint16_t*, kb, k_res, k_res) + bi * BLOCK_I64(kb, k_res, kres_sb) + hk * BLOCK_I64(kb, k_res, kres_sh);
-    W.vr = BLOCK_PTR(const uint16_t*, kb, k_res, v_res) + bi * BLOCK_I64(kb, k_res, vres_sb) + hk * BLOCK_I64(kb, k_res, vres_sh);
+    W.kr = BLOCK_PTR(const uint16_t*, kb, k_res, k_res) + bi * BLOCK_I64(kb, k_res, kres_sb) +
+           hk * BLOCK_I64(kb, k_res, kres_sh);
+    W.vr = BLOCK_PTR(const uint16_t*, kb, k_res, v_res) + bi * BLOCK_I64(kb, k_res, vres_sb) +
+           hk * BLOCK_I64(kb, k_res, vres_sh);
     W.k_st = BLOCK_I64(kb, k_res, kres_st);
     W.v_st = BLOCK_I64(kb, k_res, vres_st);
     W.kn = W.vn = nullptr;
