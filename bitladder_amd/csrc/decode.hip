@@ -169,6 +169,9 @@ __device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
 __device__ __forceinline__ float partner(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
 }
+__device__ __forceinline__ uint32_t partner(uint32_t x) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x128, 0xf, 0xf, false));
+}
 // max over the four lanes that share a column (lane, lane^16, lane^32, lane^48).
 // v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of
 // its second one, v_permlane32_swap does the same with 32-lane halves; fed two copies of x they
@@ -194,12 +197,14 @@ struct WaveState {
 
 // Online-softmax step over N raw scores t (q.k units); on return t holds
 // p = 2^kPShift * exp2(scale * (t - running max)).  Accumulators are rescaled only when the
-// running max of some head moved (wave-uniform branch).
-template <int N, int NCG>
+// running max of some head moved (wave-uniform branch).  With HALVES the hi column and the lo
+// column of a head hold different halves of the step's scores, and the maximum is taken over both.
+template <int N, int NCG, bool HALVES = false>
 __device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st) {
     float mx = t[0];
 #pragma unroll
     for (int i = 1; i < N; ++i) mx = fmaxf(mx, t[i]);
+    if constexpr (HALVES) mx = fmaxf(mx, partner(mx));
     mx = colmax(mx);
     const float m_new = fmaxf(st.m, mx);
     const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
@@ -215,6 +220,81 @@ __device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveSta
     const float c0 = kPShift - m_use * scale;
 #pragma unroll
     for (int i = 0; i < N; ++i) t[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(t[i], scale, c0));
+}
+
+// Accumulators of the four S^T tiles of a 64-token step -> probabilities as operands of the second
+// product, per 32-token sub-block ks: p16 (every column), pz (p in the hi columns, 0 in the lo ones),
+// pm (the reverse).  Element i = 4*T + r of a sub-block is tile 2*ks + T, accumulator register r.
+// A tile's hi and lo columns hold the two parts of its scores; their sum is the score.
+//
+// Plain form: every lane adds up the 16 scores of its head and takes the 16 exponentials, the lo
+// column repeating what the hi column does.
+template <int NCG>
+__device__ __forceinline__ void step_probabilities(const f4 (&sc)[4], uint32_t hi_cols, float scale, WaveState<NCG>& st,
+                                                   h8 (&p16)[2], h8 (&pz)[2], h8 (&pm)[2]) {
+    float t[16];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) t[4 * tt + r] = sc[tt][r] + partner(sc[tt][r]);
+    }
+    softmax_step<16, NCG>(t, scale, st);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        u4 pw;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            pw[x] = __builtin_bit_cast(uint32_t, pk_rtz(t[8 * ks + 2 * x], t[8 * ks + 2 * x + 1]));
+        }
+        p16[ks] = __builtin_bit_cast(h8, pw);
+        pz[ks] = __builtin_bit_cast(h8, pw & hi_cols);
+        pm[ks] = __builtin_bit_cast(h8, pw & ~hi_cols);
+    }
+}
+// Shared form, same values: the hi column takes sub-block 0 and the lo column sub-block 1 (eight sums
+// and exponentials per lane instead of sixteen), and the packed probabilities are exchanged
+// afterwards.  The sums of sub-block 0 are made in every lane; DPP adds that write only the two
+// upper banks of each row of 16 lanes then put the sums of sub-block 1 over them in the lo columns.
+// The compiler does not see that the asm reads MFMA results: the block takes all of them as operands,
+// so that it comes after the last MFMA, and waits out the longest MFMA-to-VALU distance itself.
+// Pays where a wave works through many units (1.5-2 % at 2 bits), not with one 4-bit unit per wave.
+template <int NCG>
+__device__ __forceinline__ void step_probabilities_shared(const f4 (&sc)[4], uint32_t hi_cols, float scale,
+                                                          WaveState<NCG>& st, h8 (&p16)[2], h8 (&pz)[2],
+                                                          h8 (&pm)[2]) {
+    float t[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = sc[i / 4][i % 4] + partner(sc[i / 4][i % 4]);
+    asm volatile("s_nop 7\n\ts_nop 3\n\t"
+                 "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc"
+                 : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7])
+                 : "v"(sc[2][0]), "v"(sc[2][1]), "v"(sc[2][2]), "v"(sc[2][3]), "v"(sc[3][0]), "v"(sc[3][1]),
+                   "v"(sc[3][2]), "v"(sc[3][3]));
+    softmax_step<8, NCG, true>(t, scale, st);
+    u4 pw;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) pw[x] = __builtin_bit_cast(uint32_t, pk_rtz(t[2 * x], t[2 * x + 1]));
+    const u4 z0 = pw & hi_cols;       // the hi columns hold sub-block 0
+    const u4 m1 = pw & ~hi_cols;      // the lo columns hold sub-block 1
+    u4 z1, m0;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        z1[x] = partner(m1[x]);
+        m0[x] = partner(z0[x]);
+    }
+    pz[0] = __builtin_bit_cast(h8, z0);
+    pm[0] = __builtin_bit_cast(h8, m0);
+    pz[1] = __builtin_bit_cast(h8, z1);
+    pm[1] = __builtin_bit_cast(h8, m1);
+    p16[0] = __builtin_bit_cast(h8, z0 | m0);
+    p16[1] = __builtin_bit_cast(h8, z1 | m1);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -500,7 +580,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
         wait_vm<4 - RPS + C::VSIDE>();
         if (step > 0) wait_vm<C::VSIDE>();
         PHASE(9 + 3 * step);
-        float t[4 * TPS];
+        f4 sc[TPS];
 #pragma unroll
         for (int tt = 0; tt < TPS; ++tt) {
             const int tile = step * TPS + tt;
@@ -522,8 +602,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
                     acc = mfma32(a1, G.qp[2 * jj + 1], acc);
                 }
             }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) t[4 * tt + r] = acc[r] + partner(acc[r]);   // hi + lo
+            sc[tt] = acc;
         }
         // every K row and this unit's K parameters have been read: the next unit's K side may land
         if (HAS_NEXT && step == kLast) {
@@ -532,22 +611,15 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
         }
         PHASE(10 + 3 * step);
 
-        softmax_step<4 * TPS, NCG>(t, P.scale_log2, st);
-
+        static_assert(TPS == 4 && NKS == 2, "four tiles, two sub-blocks per step");
         h8 p16[NKS], pz[NKS], pm[NKS];
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-            u4 pw;
-#pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                // element i = 4*T + r  <->  tile 2*ks + T of the step, accumulator register r
-                pw[x] = __builtin_bit_cast(uint32_t, pk_rtz(t[8 * ks + 2 * x], t[8 * ks + 2 * x + 1]));
-            }
-            p16[ks] = __builtin_bit_cast(h8, pw);
-            pz[ks] = __builtin_bit_cast(h8, pw & hi_cols);       // p itself only in the hi columns
-            pm[ks] = __builtin_bit_cast(h8, pw & ~hi_cols);      // and only in the lo columns
-            st.l = mfma32(ones, pz[ks], st.l);
+        if constexpr (BITS == 2) {
+            step_probabilities_shared<NCG>(sc, hi_cols, P.scale_log2, st, p16, pz, pm);
+        } else {
+            step_probabilities<NCG>(sc, hi_cols, P.scale_log2, st, p16, pz, pm);
         }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) st.l = mfma32(ones, pz[ks], st.l);
         PHASE(11 + 3 * step);
         // still allowed in flight: the V rows of later steps and, once issued, the next unit's K side
         wait_vm_n((HAS_NEXT && step == kLast) ? C::KSIDE : 4 - (step + 1) * RPS);
