@@ -169,8 +169,10 @@ __device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
 __device__ __forceinline__ float partner(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
 }
+// (every lane has a source lane, so the "bound control" flag changes nothing but tells the compiler
+// that no previous value of the result survives, which saves it a move)
 __device__ __forceinline__ uint32_t partner(uint32_t x) {
-    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x128, 0xf, 0xf, false));
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x128, 0xf, 0xf, true));
 }
 // max over the four lanes that share a column (lane, lane^16, lane^32, lane^48).
 // v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of
@@ -200,10 +202,7 @@ struct WaveState {
 // running max of some head moved (wave-uniform branch).  With HALVES the hi column and the lo
 // column of a head hold different halves of the step's scores, and the maximum is taken over both.
 template <int N, int NCG, bool HALVES = false>
-__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st) {
-    float mx = t[0];
-#pragma unroll
-    for (int i = 1; i < N; ++i) mx = fmaxf(mx, t[i]);
+__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st, float mx) {
     if constexpr (HALVES) mx = fmaxf(mx, partner(mx));
     mx = colmax(mx);
     const float m_new = fmaxf(st.m, mx);
@@ -220,6 +219,13 @@ __device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveSta
     const float c0 = kPShift - m_use * scale;
 #pragma unroll
     for (int i = 0; i < N; ++i) t[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(t[i], scale, c0));
+}
+template <int N, int NCG>
+__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st) {
+    float mx = t[0];
+#pragma unroll
+    for (int i = 1; i < N; ++i) mx = fmaxf(mx, t[i]);
+    softmax_step<N, NCG>(t, scale, st, mx);
 }
 
 // Accumulators of the four S^T tiles of a 64-token step -> probabilities as operands of the second
@@ -257,7 +263,7 @@ __device__ __forceinline__ void step_probabilities(const f4 (&sc)[4], uint32_t h
 // upper banks of each row of 16 lanes then put the sums of sub-block 1 over them in the lo columns.
 // The compiler does not see that the asm reads MFMA results: the block takes all of them as operands,
 // so that it comes after the last MFMA, and waits out the longest MFMA-to-VALU distance itself.
-// Pays where a wave works through many units (1.5-2 % at 2 bits), not with one 4-bit unit per wave.
+// Pays where a wave works through many units (2-4 % at 2 bits), not with one 4-bit unit per wave.
 template <int NCG>
 __device__ __forceinline__ void step_probabilities_shared(const f4 (&sc)[4], uint32_t hi_cols, float scale,
                                                           WaveState<NCG>& st, h8 (&p16)[2], h8 (&pz)[2],
@@ -265,19 +271,25 @@ __device__ __forceinline__ void step_probabilities_shared(const f4 (&sc)[4], uin
     float t[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) t[i] = sc[i / 4][i % 4] + partner(sc[i / 4][i % 4]);
+    float mx;      // maximum of the lane's eight sums
     asm volatile("s_nop 7\n\ts_nop 3\n\t"
-                 "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                 "v_add_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc"
-                 : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7])
+                 "v_add_f32_dpp %0, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %1, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %2, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %3, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %4, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %5, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %6, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_add_f32_dpp %7, %16, %16 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                 "v_max3_f32 %8, %0, %1, %2\n\t"
+                 "v_max3_f32 %8, %8, %3, %4\n\t"
+                 "v_max3_f32 %8, %8, %5, %6\n\t"
+                 "v_max_f32 %8, %8, %7"
+                 : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]),
+                   "=&v"(mx)
                  : "v"(sc[2][0]), "v"(sc[2][1]), "v"(sc[2][2]), "v"(sc[2][3]), "v"(sc[3][0]), "v"(sc[3][1]),
                    "v"(sc[3][2]), "v"(sc[3][3]));
-    softmax_step<8, NCG, true>(t, scale, st);
+    softmax_step<8, NCG, true>(t, scale, st, mx);
     u4 pw;
 #pragma unroll
     for (int x = 0; x < 4; ++x) pw[x] = __builtin_bit_cast(uint32_t, pk_rtz(t[2 * x], t[2 * x + 1]));
