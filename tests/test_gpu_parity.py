@@ -266,7 +266,8 @@ def test_qpack_ranges_from_subnormal_to_max(device, bits, dtype):
     H.assert_cache_equals_oracle(H.cache_to_numpy(*cache), want)
 
 
-@pytest.mark.parametrize("bits,gs,S,ns", [(4, 32, 4096, 1), (4, 32, 8192, 2), (4, 128, 8192, 1), (2, 64, 16384, 1)])
+@pytest.mark.parametrize("bits,gs,S,ns", [(4, 32, 4096, 1), (4, 32, 8192, 2), (4, 128, 8192, 1), (2, 64, 16384, 1),
+                                        (2, 128, 16384, 1), (2, 32, 8192, 1), (2, 128, 16384, 2)])
 def test_waves_with_many_units_on_cache_resident_data_are_deterministic(device, bits, gs, S, ns):
     """Each wave streams three or more units through its LDS region, and the cache is small enough to stay in
     L2 while the call is repeated: the direct-to-LDS loads of the next unit then come back fast, and must
