@@ -80,8 +80,8 @@ int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t m
     return choose_splits(b, h_k, max_seqlen_k, max_res_len, num_cus, bits, group_size);
 }
 
-// [tickets: b*h ints rounded up to 256 B][o_part][ml_part]
-static size_t ticket_bytes(int32_t b, int32_t h) { return (static_cast<size_t>(b) * h * sizeof(int) + 255) / 256 * 256; }
+// [tickets: one 256-byte block per (batch, query head)][o_part][ml_part]
+static size_t ticket_bytes(int32_t b, int32_t h) { return static_cast<size_t>(b) * h * bitdecode::kTicketStride * sizeof(int); }
 
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     if (num_splits <= 1) return 0;
@@ -160,7 +160,7 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
 }
 
 // bytes of the per-sequence step counters that lead a step workspace
-static size_t step_ticket_bytes(int32_t b) { return (static_cast<size_t>(b) * sizeof(int) + 255) / 256 * 256; }
+static size_t step_ticket_bytes(int32_t b) { return static_cast<size_t>(b) * bitdecode::kTicketStride * sizeof(int); }
 
 size_t bitdecode_fwd_append_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     return step_ticket_bytes(b) + bitdecode_fwd_workspace_bytes(b, h, num_splits);

@@ -562,7 +562,7 @@ __device__ __forceinline__ void start_group(KGroup& G, const uint8_t* kpar, cons
 // scale is applied inside the exponent.  On entry both sides of the unit are in flight or landed
 // (queue order: K side, V side).  With HAS_NEXT the two sides of the wave's next unit are issued
 // from here (see above); kslot says which K-parameter slot the current unit uses.
-template <int BITS, int GS, bool BF16, bool HAS_NEXT>
+template <int BITS, int GS, bool BF16, bool HAS_NEXT, bool DEFER_V = false>
 __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, int kslot,
                                              const UnitAddr<BITS, GS>& next, const QRows& Q, const FwdParams& P,
                                              int lane, bool lo_part, const Magic& mg, WaveState<kHeadDim / GS>& st,
@@ -579,8 +579,10 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     const uint8_t* kpar = reg + C::OFF_KP + kslot * C::KPB;
     const uint8_t* vpar = reg + C::OFF_VP + kg * 16;
 
+    static_assert(!(HAS_NEXT && DEFER_V), "only a wave's single unit defers its V side");
     // the K parameters lead the queue: the first K group is prepared while the code rows arrive
-    wait_vm<4 + C::VSIDE>();
+    constexpr int VQ0 = DEFER_V ? 0 : C::VSIDE;      // V-side loads behind the K side while step 0 runs
+    wait_vm<4 + VQ0>();
     PHASE(8);
     KGroup G;
     start_group<BITS, BF16>(G, kpar, Q, kg);
@@ -589,7 +591,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     for (int step = 0; step < NSTEP; ++step) {
         constexpr int kLast = NSTEP - 1;
         // still allowed in flight: the K rows of later steps and the whole V side
-        wait_vm<4 - RPS + C::VSIDE>();
+        wait_vm<4 - RPS + VQ0>();
         if (step > 0) wait_vm<C::VSIDE>();
         PHASE(9 + 3 * step);
         f4 sc[TPS];
@@ -632,37 +634,59 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
         }
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) st.l = mfma32(ones, pz[ks], st.l);
+        if (DEFER_V && step == 0) {
+#ifdef X_PRIO
+            __builtin_amdgcn_s_setprio(0);
+#endif
+            issue_vside<BITS, GS>(next, lane * 16, region_lds);      // `next` is this unit here
+        }
         PHASE(11 + 3 * step);
-        // still allowed in flight: the V rows of later steps and, once issued, the next unit's K side
-        wait_vm_n((HAS_NEXT && step == kLast) ? C::KSIDE : 4 - (step + 1) * RPS);
+        // V side of the step, row by row in the order the rows arrive.  A row holds one channel half
+        // (tiles ct = 4*hf .. 4*hf+3) of one 32-token sub-block (4 bits) or of the whole step (2 bits).
+        // Still allowed in flight behind row r of the unit: the rows after it and, once issued, the
+        // next unit's K side.  A wave's last unit waits row by row, so that only the products of the
+        // last row are left when the last byte lands; a unit with a successor waits once per step.
+        constexpr int kNextK = HAS_NEXT ? C::KSIDE : 0;
+        const int behind = (step == kLast) ? kNextK : 0;
+        if constexpr (HAS_NEXT) {
+            wait_vm_n(behind + 4 - (step + 1) * RPS);
+        } else if (step == 0) {
+            wait_vm<4>();              // the V parameters
+        }
+        h8 pp[NCG][NKS];
+        constexpr int CGH = NCG >= 2 ? NCG / 2 : 1;      // channel groups per channel half
 #pragma unroll
-        for (int cg = 0; cg < NCG; ++cg) {
-            h8 pp[NKS];
+        for (int r = 0; r < RPS; ++r) {
+            const int hf = r % 2;
+            const int ksr = (BITS == 4) ? r / 2 : 0;     // 4 bits: the row's sub-block
+            // p * scale (exact hi/lo pair) and the bias terms of the channel groups this row starts
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                const int sb = step * NKS + ks;               // 32-token sub-block inside the unit
-                const u4 rs = *reinterpret_cast<const u4*>(vpar + (sb * NCG + cg) * 128);
-                const u4 rz = *reinterpret_cast<const u4*>(vpar + (sb * NCG + cg) * 128 + 64);
-                pp[ks] = split_mul_masked(p16[ks], pm[ks], cvt_h8<false>(rs));
-                st.ob[cg] = mfma32(cvt_h8<false>(rz), pz[ks], st.ob[cg]);
-                st.ob[cg] = mfma32(noff, pp[ks], st.ob[cg]);
-            }
+            for (int c = 0; c < CGH; ++c) {
+                const int cg = NCG >= 2 ? hf * CGH + c : 0;
+                if (NCG >= 2 || hf == 0) {
 #pragma unroll
-            for (int x = 0; x < CTPG; ++x) {
-                const int ct = cg * CTPG + x;
-                if constexpr (BITS == 4) {
-                    // rows of the step: (sub-block ks, channel half ct / 4)
-#pragma unroll
-                    for (int ks = 0; ks < NKS; ++ks) {
-                        const uint32_t w = vcode[64 * (2 * ks + ct / 4)][ct & 3];
-                        st.o[ct] = mfma32(dq4(w, mg), pp[ks], st.o[ct]);
+                    for (int ks = (BITS == 4 ? ksr : 0); ks < (BITS == 4 ? ksr + 1 : NKS); ++ks) {
+                        const int sb = step * NKS + ks;               // 32-token sub-block inside the unit
+                        const u4 rs = *reinterpret_cast<const u4*>(vpar + (sb * NCG + cg) * 128);
+                        const u4 rz = *reinterpret_cast<const u4*>(vpar + (sb * NCG + cg) * 128 + 64);
+                        pp[cg][ks] = split_mul_masked(p16[ks], pm[ks], cvt_h8<false>(rs));
+                        st.ob[cg] = mfma32(cvt_h8<false>(rz), pz[ks], st.ob[cg]);
+                        st.ob[cg] = mfma32(noff, pp[cg][ks], st.ob[cg]);
                     }
+                }
+            }
+            if constexpr (!HAS_NEXT) wait_vm_n(3 - (step * RPS + r));
+            const u4 w = vcode[64 * (step * RPS + r)];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int ct = 4 * hf + x, cg = ct / CTPG;
+                if constexpr (BITS == 4) {
+                    st.o[ct] = mfma32(dq4(w[x], mg), pp[cg][ksr], st.o[ct]);
                 } else {
-                    const uint32_t w = vcode[64 * (2 * step + ct / 4)][ct & 3];
                     h8 a0, a1;
-                    dq2(w, a0, a1, mg);
-                    st.o[ct] = mfma32(a0, pp[0], st.o[ct]);
-                    st.o[ct] = mfma32(a1, pp[1], st.o[ct]);
+                    dq2(w[x], a0, a1, mg);
+                    st.o[ct] = mfma32(a0, pp[cg][0], st.o[ct]);
+                    st.o[ct] = mfma32(a1, pp[cg][1], st.o[ct]);
                 }
             }
         }
@@ -839,49 +863,105 @@ __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P,
     }
 }
 
-// device-scope (agent) relaxed accesses: write-through stores / cache-coherent loads
-__device__ __forceinline__ void st_dev(float* p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// device-scope (agent) relaxed accesses of 8 bytes: write-through stores / loads served from the
+// level all compute units share
+__device__ __forceinline__ void st_dev2(float* p, float a, float b) {
+    const uint64_t bits = __float_as_uint(a) | (static_cast<uint64_t>(__float_as_uint(b)) << 32);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ float ld_dev(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ float2 ld_dev2(const float* p) {
+    const uint64_t bits = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return float2{__uint_as_float(static_cast<uint32_t>(bits)), __uint_as_float(static_cast<uint32_t>(bits >> 32))};
 }
 
-// partial outputs of splits s0 .. s0+31 (clamped to the last split) for one (head, channel).  The
-// split's base address is wave-uniform (SGPRs) and `item` a 32-bit per-thread offset, so the 32
-// loads need no per-load address arithmetic.
-__device__ __forceinline__ void load_partials(float (&v)[32], const float* o_part, uint32_t item, int64_t split_stride,
-                                              int s0, int nsplit) {
-    const float* base = o_part + static_cast<int64_t>(s0) * split_stride;
+// x of lane `l` (wave-uniform index) as a scalar
+__device__ __forceinline__ float lane_value(float x, int l) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l));
+}
+// DPP row rotation: value of lane (l + N) % 16 of the same row of 16 lanes
+template <int N>
+__device__ __forceinline__ float row_ror(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + N, 0xf, 0xf, true));
+}
+// reductions over each row of 16 lanes, result in every lane of the row; the additions are grouped the
+// same way in every run
+__device__ __forceinline__ float row_max16(float x) {
+    x = fmaxf(x, row_ror<8>(x));
+    x = fmaxf(x, row_ror<4>(x));
+    x = fmaxf(x, row_ror<2>(x));
+    return fmaxf(x, row_ror<1>(x));
+}
+__device__ __forceinline__ float row_sum16(float x) {
+    x += row_ror<8>(x);
+    x += row_ror<4>(x);
+    x += row_ror<2>(x);
+    return x + row_ror<1>(x);
+}
+// the same over the whole wave, as a scalar
+__device__ __forceinline__ float wave_max(float x) {
+    x = row_max16(x);
+    return fmaxf(fmaxf(lane_value(x, 0), lane_value(x, 16)), fmaxf(lane_value(x, 32), lane_value(x, 48)));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+    x = row_sum16(x);
+    return (lane_value(x, 0) + lane_value(x, 16)) + (lane_value(x, 32) + lane_value(x, 48));
+}
+
+// partial outputs (two channels per lane) of splits s0 .. s0+31, clamped to the last split
+__device__ __forceinline__ void load_partials(float2 (&v)[32], const float* base, int64_t split_stride, int s0, int nsplit) {
+    base += static_cast<int64_t>(s0) * split_stride;
     const int cnt = min(32, nsplit - s0);
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
-        v[k] = ld_dev(base + item);
+        v[k] = ld_dev2(base);
         if (k + 1 < cnt) base += split_stride;
     }
 }
-// (maximum, sum) pairs of splits s0 + s8 + 8k, k = 0..7 (clamped to the last split), for one head
-__device__ __forceinline__ void load_ml(float (&m)[8], float (&l)[8], const float* ml_part, int64_t row,
-                                        int64_t split_stride, int s0, int s8, int nsplit) {
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        const int sp = min(s0 + s8 + 8 * k, nsplit - 1);
-        const float* src = ml_part + 2 * (sp * split_stride + row);
-        m[k] = ld_dev(src);
-        l[k] = ld_dev(src + 1);
-    }
-}
 
-// reductions over the eight lanes that share lane % 8 (one head), in a fixed butterfly order
-__device__ __forceinline__ float head_max(float x) {
-    x = fmaxf(x, __shfl_xor(x, 8));
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
-}
-__device__ __forceinline__ float head_sum(float x) {
-    x += __shfl_xor(x, 8);
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
+// Merge of the splits of one query head by one wave (flash_fwd_kernel.h:1217-1298 in unnormalised
+// form): out = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M).  Lane l owns channels 2l and
+// 2l+1; the (M, L) pairs are spread over the lanes (split s0 + l of each round of 64), the weights go
+// back to all lanes as scalars.  The order of the additions is fixed.
+__device__ __forceinline__ void merge_splits(const float* o_part, const float* ml_part, int64_t hrow, int64_t hstride,
+                                             int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
+    const float* ob = o_part + hrow * kHeadDim + 2 * lane;
+    const int64_t sstride = hstride * kHeadDim;
+    const float* mlb = ml_part + hrow * nsplit * 2;
+    const float2 none = float2{-INFINITY, 0.0f};
+    const float2 ml0 = lane < nsplit ? ld_dev2(mlb + 2 * lane) : none;      // ahead of the bulk loads
+    float2 v[32];
+    load_partials(v, ob, sstride, 0, nsplit);
+    float mx = ml0.x;
+    for (int sb = 64; sb < nsplit; sb += 64) {
+        if (sb + lane < nsplit) mx = fmaxf(mx, ld_dev2(mlb + 2 * (sb + lane)).x);
+    }
+    M = wave_max(mx);
+    const float Mu = (M == -INFINITY) ? 0.0f : M;
+    float lacc = 0.0f;
+    O0 = O1 = 0.0f;
+    for (int sb = 0; sb < nsplit; sb += 64) {
+        float2 ml = ml0;
+        if (sb > 0) ml = sb + lane < nsplit ? ld_dev2(mlb + 2 * (sb + lane)) : none;
+        const float w = __builtin_amdgcn_exp2f(ml.x - Mu);       // 0 past the last split
+        lacc = __builtin_fmaf(w, ml.y, lacc);
+        if (sb > 0) load_partials(v, ob, sstride, sb, nsplit);
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const float wk = lane_value(w, k);
+            O0 = __builtin_fmaf(wk, v[k].x, O0);
+            O1 = __builtin_fmaf(wk, v[k].y, O1);
+        }
+        if (sb + 32 < nsplit) {
+            load_partials(v, ob, sstride, sb + 32, nsplit);
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                const float wk = lane_value(w, 32 + k);
+                O0 = __builtin_fmaf(wk, v[k].x, O0);
+                O1 = __builtin_fmaf(wk, v[k].y, O1);
+            }
+        }
+    }
+    L = wave_sum(lacc);
 }
 
 template <bool BF16>
@@ -894,6 +974,21 @@ __device__ __forceinline__ uint16_t to_out(float f) {
     } else {
         return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
     }
+}
+
+// Final values of one query head: lane l writes channels 2l, 2l+1 of O / L, lane 0 the natural-log LSE
+// (softmax.h:303; +inf for a row without keys).
+template <bool BF16>
+__device__ __forceinline__ void write_head(uint16_t* out_row, float* lse, int lane, float O0, float O1, float M, float L) {
+    const bool none = !(L > 0.0f);
+    const uint16_t a = to_out<BF16>(none ? 0.0f : O0 / L), b = to_out<BF16>(none ? 0.0f : O1 / L);
+    if ((reinterpret_cast<uintptr_t>(out_row) & 3u) == 0) {
+        reinterpret_cast<uint32_t*>(out_row)[lane] = a | (static_cast<uint32_t>(b) << 16);
+    } else {
+        out_row[2 * lane] = a;
+        out_row[2 * lane + 1] = b;
+    }
+    if (lane == 0 && lse) *lse = none ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -913,10 +1008,10 @@ __device__ __forceinline__ bool step_overflows(int capacity, int t) {
 // the last of the h_k tickets of a sequence knows that every workgroup of the sequence has read the
 // length, advances it and resets the counter.
 __device__ __forceinline__ void step_ticket(int* step_tickets, int* lengths, int n_heads_k, int capacity, int bi, int t) {
-    const int drawn = __hip_atomic_fetch_add(&step_tickets[bi], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int drawn = __hip_atomic_fetch_add(&step_tickets[bi * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (drawn == n_heads_k - 1) {
         // read again only by the next launch: plain stores
-        step_tickets[bi] = 0;
+        step_tickets[bi * kTicketStride] = 0;
         if (!step_overflows(capacity, t)) lengths[bi] = t + 1;
     }
 }
@@ -985,15 +1080,13 @@ __device__ __forceinline__ void step_end(uint8_t* lds, int bi, int hk, int t) {
 // (flash_fwd_kernel.h:1217-1298 formula) and resets the ticket.
 //
 // Dynamic LDS: [NW wave regions of UnitCfg::REGION bytes][q: 8 head rows + a zero row, 272 B apart]
-// [sM, sL: per-wave max and sum, NW x 8 floats each][sA: merge weights, 8 x NW][sHead: merged max and
-// sum, 2 x 8][last-ticket flag].  A wave's region is reused as its V-transpose slab for fp16 tiles
-// and as its slot of the cross-wave merge buffer (g x 128 floats <= 4 KB); the merging workgroup
-// reuses the regions for the per-split maxima, sums and weights.
+// [sM, sL: per-wave max and sum, 8 heads x NW floats each][append flag].  A wave's region is reused as its
+// V-transpose slab for fp16 tiles and as its slot of the cross-wave merge buffer (g x 128 floats <= 4 KB).
 // ---------------------------------------------------------------------------------------------
 template <int BITS, int GS>
 constexpr int fwd_lds_bytes() {
     using C = UnitCfg<BITS, GS>;
-    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + (3 * C::NW + 2) * kMaxGroupHeads * 4 + 16;
+    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16;
 }
 
 template <int BITS, int GS, bool BF16, bool APPEND>
@@ -1003,11 +1096,9 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     static_assert(sizeof(qp::PackLds<GS>) <= NW * REGION, "the pack tile reuses the wave regions");
     uint8_t* const sq = lds + NW * REGION;                                   // [8 + zero row][128] 16-bit q
-    float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * kQRowBytes);   // [NW][8]
+    float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * kQRowBytes);   // [8][NW]
     float* const sL = sM + NW * kMaxGroupHeads;
-    float* const sA = sL + NW * kMaxGroupHeads;                                   // [8][NW] merge weights
-    float* const sHead = sA + NW * kMaxGroupHeads;                                // [2][8] merged max, sum
-    int* const s_last = reinterpret_cast<int*>(sHead + 2 * kMaxGroupHeads);
+    int* const s_last = reinterpret_cast<int*>(sL + NW * kMaxGroupHeads);
 
     PROF_DECL;
     PROF(0);
@@ -1068,12 +1159,29 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         qa_raw = load_untracked(q0 + (hq < g ? hq : 0) * P.q_sh);
         qb_raw = load_untracked(q0 + (hq + 4 < g ? hq + 4 : 0) * P.q_sh);
     }
+    // First units: every wave of the workgroup sends out its K side before any wave sends its V side
+    // (loads come back roughly in the order the compute unit issued them).  The K sides then land in
+    // the first half of the stream and the scores and probabilities of all waves are ready while the V
+    // sides are still arriving: after the last byte only the products of the last V row are left.
+    // (A bare s_barrier: no wait for the loads in flight.)
     UnitAddr<BITS, GS> A;
+#ifdef X_DEFERV
+    const bool single = u + NW >= u1;      // at most one packed unit for this wave
+#else
+    const bool single = false;
+#endif
     if (u < u1) {
+#ifdef X_PRIO
+        __builtin_amdgcn_s_setprio(3);
+#endif
         A = unit_addr<BITS, GS>(P, bi, hk, u);
         issue_kside<BITS, GS>(A, lane * 16, region_lds, 0);
-        issue_vside<BITS, GS>(A, lane * 16, region_lds);
-        wait_then_take<C::KSIDE + C::VSIDE>(qa, qb, qa_raw, qb_raw);
+        if (!single) {
+            issue_vside<BITS, GS>(A, lane * 16, region_lds);
+            wait_then_take<C::KSIDE + C::VSIDE>(qa, qb, qa_raw, qb_raw);
+        } else {
+            wait_then_take<C::KSIDE>(qa, qb, qa_raw, qb_raw);
+        }
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
     }
@@ -1106,7 +1214,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     if (u < u1) {
         const Magic mg;
 #ifdef BITDECODE_PROF
-        wait_vm<4 + C::VSIDE>();   // K parameters have arrived
+        if (single) wait_vm<4>(); else wait_vm<4 + C::VSIDE>();   // K parameters have arrived
         PROF(2);
         unsigned long long* phase_ts = prof_ts;
 #else
@@ -1119,7 +1227,11 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
             kslot ^= 1;
             phase_ts = nullptr;
         }
-        compute_unit<BITS, GS, BF16, false>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
+        if (single) {     // (the wave's only unit: its V side is still to be issued)
+            compute_unit<BITS, GS, BF16, false, true>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
+        } else {
+            compute_unit<BITS, GS, BF16, false>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
+        }
     }
     PROF(3);
     // ---- fp16 window tiles of this wave (the region becomes the V-transpose slab)
@@ -1161,38 +1273,34 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         }
     }
     if (kg == 0 && col < kMaxGroupHeads) {
-        sM[wave * kMaxGroupHeads + col] = col < g ? st.m * P.scale_log2 : -INFINITY;     // base-2 units
-        sL[wave * kMaxGroupHeads + col] = col < g ? lsum : 0.0f;
+        sM[col * NW + wave] = col < g ? st.m * P.scale_log2 : -INFINITY;     // base-2 units
+        sL[col * NW + wave] = col < g ? lsum : 0.0f;
     }
     __syncthreads();
     PROF(4);
     if constexpr (APPEND) {
         if (P.nsplit == 1) step_begin<NW>(bi, hk, step_len);     // a single split: every wave is past the window
     }
-    // one wave turns the per-wave maxima and sums into weights: lane (w8, head) covers waves w8, w8 + 8
-    if (wave == 0) {
-        const int hh = lane & 7, w8 = lane >> 3;
-        const bool two = w8 + 8 < NW;
-        const float m0 = sM[w8 * kMaxGroupHeads + hh];
-        const float m1 = two ? sM[(w8 + 8) * kMaxGroupHeads + hh] : -INFINITY;
-        const float M = head_max(fmaxf(m0, m1));
-        const float Mu = (M == -INFINITY) ? 0.0f : M;
-        const float a0 = __builtin_amdgcn_exp2f(m0 - Mu), a1 = __builtin_amdgcn_exp2f(m1 - Mu);
-        sA[hh * NW + w8] = a0;
-        float L = a0 * sL[w8 * kMaxGroupHeads + hh];
-        if (two) {
-            sA[hh * NW + w8 + 8] = a1;
-            L += a1 * sL[(w8 + 8) * kMaxGroupHeads + hh];
-        }
-        L = head_sum(L);
-        if (w8 == 0) {
-            sHead[hh] = M;
-            sHead[kMaxGroupHeads + hh] = L;
-        }
-    }
-    __syncthreads();
-    // the workgroup's result relative to its own maximum: O = sum_w a_w O_w, with (M, L) per head.
-    // A single split normalises and writes the output; otherwise the triple is published as is.
+    // From here on wave hh < g works alone on query head hh of the group, lane l on channels 2l and 2l+1;
+    // nothing below needs another workgroup barrier (the decode step with append has one, to elect the
+    // workgroup that appends).
+    //
+    // Protocol between the splits of one query head (workspace: counters, partial outputs, (max, sum)
+    // pairs; all in ordinary device memory):
+    //  1. a wave writes its head's partial output and (max, sum) with device-scope write-through stores;
+    //  2. it waits until all its stores are acknowledged (s_waitcnt vmcnt(0)): they are then visible to
+    //     device-scope loads of any compute unit;
+    //  3. one lane draws a ticket from the head's counter with a device-scope atomic add (performed at the
+    //     memory side, so tickets of different compute units are totally ordered);
+    //  4. the wave whose ticket is the last one knows that every other split passed step 2 before its
+    //     step 3; it resets the counter (read again only by the next launch on this workspace) and reads
+    //     all partials with device-scope loads, which are served from the coherent level and not from a
+    //     stale line of its own caches.
+    // The asm waits are compiler barriers ("memory" clobber), so neither the stores nor the loads move
+    // across the ticket.  What would break it: a workspace in host-coherent or fine-grained memory with
+    // other scope rules, two launches in flight on one workspace, or non-zero counters at the first launch.
+    bool last = false;
+    float O0 = 0.0f, O1 = 0.0f, M = -INFINITY, L = 0.0f;
     uint16_t* out = P.out;
     int64_t out_sb = P.out_sb, out_sh = P.out_sh;
     float* lse_out = P.lse;
@@ -1212,141 +1320,65 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         n_h = BLOCK_I32(ob, o_part, h);
         n_b = BLOCK_I32(ob, o_part, b);
     }
+    const int hq = hk * g + wave;                                  // this wave's query head
+    const int64_t hrow = static_cast<int64_t>(bi) * n_h + hq;      // its row in [b][h] tables
     const int64_t hstride = static_cast<int64_t>(n_b) * n_h;       // rows per split in the workspace
-    for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
-        const int hh = idx >> 7, c = idx & 127;
-        float aw[NW];      // NW is a multiple of 4: four weights per LDS read
-#pragma unroll
-        for (int w = 0; w < NW; w += 4) {
-            const f4 a4 = *reinterpret_cast<const f4*>(&sA[hh * NW + w]);
-            aw[w] = a4[0]; aw[w + 1] = a4[1]; aw[w + 2] = a4[2]; aw[w + 3] = a4[3];
-        }
-        float O = 0.0f;
+    uint16_t* const out_row = out + bi * out_sb + hq * out_sh;
+    if (wave < g) {
+        // weights of the waves: lane (any row, w) takes wave w; the row reductions give every lane the
+        // head's maximum, the weights travel to all lanes as scalars
+        const int w16 = lane & 15;
+        const float mw = w16 < NW ? sM[wave * NW + w16] : -INFINITY;
+        const float lw = w16 < NW ? sL[wave * NW + w16] : 0.0f;
+        M = row_max16(mw);
+        const float Mu = (M == -INFINITY) ? 0.0f : M;
+        const float aw = __builtin_amdgcn_exp2f(mw - Mu);
+        L = lane_value(row_sum16(aw * lw), 0);
+        const float* mine = reinterpret_cast<const float*>(lds) + wave * kHeadDim + 2 * lane;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            O += aw[w] * reinterpret_cast<const float*>(lds + w * REGION)[hh * kHeadDim + c];
+            const float a = lane_value(aw, w);
+            const float2 v = *reinterpret_cast<const float2*>(mine + w * (REGION / 4));
+            O0 = __builtin_fmaf(a, v.x, O0);
+            O1 = __builtin_fmaf(a, v.y, O1);
         }
-        const float M = sHead[hh], L = sHead[kMaxGroupHeads + hh];
-        const int hq = hk * g + hh;
         if (P.nsplit == 1) {
-            const bool empty = !(L > 0.0f);
-            out[bi * out_sb + hq * out_sh + c] = to_out<BF16>(empty ? 0.0f : O / L);
-            // natural-log LSE (softmax.h:303); +inf for a row without keys
-            if (c == 0 && lse_out) {
-                lse_out[bi * n_h + hq] = empty ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
-            }
+            write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
         } else {
-            const int64_t row = split * hstride + bi * n_h + hq;
-            st_dev(&o_part[row * kHeadDim + c], O);
-            if (c == 0) {
-                st_dev(&ml_part[2 * row], M);
-                st_dev(&ml_part[2 * row + 1], L);
+            st_dev2(&o_part[(split * hstride + hrow) * kHeadDim + 2 * lane], O0, O1);
+            if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M, L);
+            wait_vm<0>();
+            PROF(5);
+            int drawn = 0;
+            if (lane == 0) drawn = __hip_atomic_fetch_add(&tickets[hrow * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            drawn = __builtin_amdgcn_readfirstlane(drawn);
+            last = drawn == P.nsplit - 1;
+            if (last && lane == 0) __hip_atomic_store(&tickets[hrow * kTicketStride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            PROF(6);
+            if constexpr (APPEND) {
+                if (wave == 0) *s_last = last;
+            } else if (last) {
+                merge_splits(o_part, ml_part, hrow, hstride, P.nsplit, lane, O0, O1, M, L);
+                write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
             }
         }
     }
-    PROF(5);
-    if (P.nsplit > 1) {
-    // ---- the workgroup that draws the last ticket of this (batch, kv-head) merges the splits.
-    // Partials are written with device-scope (write-through) stores; once a thread's stores have
-    // completed (vmcnt 0) and the workgroup has met at the barrier, thread 0 takes the ticket.
-    // The merging workgroup reads the partials with device-scope loads, so no cache-wide
-    // write-back or invalidate is needed on either side.
-    wait_vm<0>();
-    __syncthreads();
-    if (tid == 0) {
-        const int old = __hip_atomic_fetch_add(&tickets[bh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int last = (old == P.nsplit - 1);
-        *s_last = last;
-        if (last) __hip_atomic_store(&tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    PROF(6);
-    if (!*s_last) {
-        PROF_FLUSH();
-        return;
-    }
-    if constexpr (APPEND) step_begin<NW>(bi, hk, step_len);     // every other split of the pair has finished
-    // Every thread owns one (head, channel) and starts fetching the partial outputs of the first 32
-    // splits at once; meanwhile wave 0 fetches the (M, L) pairs, lane (s8, head) taking splits
-    // s8, s8 + 8, ..., and turns them into one weight per split and head in LDS (the regions are
-    // free by now).  out = sum_s w_s O_s / sum_s w_s L_s.
-    const int nsp32 = (P.nsplit + 31) & ~31;
-    float* const tM = reinterpret_cast<float*>(lds);                  // [nsplit][8] maxima
-    float* const tL = tM + P.nsplit * kMaxGroupHeads;                  // [nsplit][8] sums
-    float* const sW = tL + P.nsplit * kMaxGroupHeads;                  // [8][nsp32] weights, zero past nsplit
-    const int64_t row00 = bi * n_h + hk * g;
-    float v0[32], m8[8], l8[8];
-    const int wl_hh = lane & 7, wl_s8 = lane >> 3;
-    const int64_t wl_row = row00 + (wl_hh < g ? wl_hh : 0);
-    if (wave == 0) load_ml(m8, l8, ml_part, wl_row, hstride, 0, wl_s8, P.nsplit);     // ahead of the bulk loads
-    if (tid < g * kHeadDim) load_partials(v0, o_part, static_cast<uint32_t>((row00 + (tid >> 7)) * kHeadDim + (tid & 127)),
-                                          hstride * kHeadDim, 0, P.nsplit);
-    PROF(12);
-    if (wave == 0) {
-        const int hh = wl_hh, s8 = wl_s8;
-        const bool live = hh < g;
-        float M = -INFINITY;
-        for (int sb = 0; sb < P.nsplit; sb += 64) {      // eight splits per lane and round
-            if (sb > 0) load_ml(m8, l8, ml_part, wl_row, hstride, sb, s8, P.nsplit);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int sp = sb + s8 + 8 * k;
-                if (sp < P.nsplit) {
-                    const float mk = live ? m8[k] : -INFINITY;
-                    tM[sp * kMaxGroupHeads + hh] = mk;
-                    tL[sp * kMaxGroupHeads + hh] = live ? l8[k] : 0.0f;
-                    M = fmaxf(M, mk);
-                }
+    if constexpr (APPEND) {
+        // The workgroup whose wave 0 drew the last ticket of the group's first head appends: every other
+        // workgroup of the (batch, kv-head) has published, so none of them reads the window or the cache
+        // any more.  Its last two waves store the token while the merging waves fetch the partials.
+        bool appends = true;
+        if (P.nsplit > 1) {
+            __syncthreads();
+            appends = *s_last != 0;
+            if (appends) step_begin<NW>(bi, hk, step_len);
+            if (wave < g && last) {
+                merge_splits(o_part, ml_part, hrow, hstride, P.nsplit, lane, O0, O1, M, L);
+                write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
             }
         }
-        M = head_max(M);
-        const float Mu = (M == -INFINITY) ? 0.0f : M;
-        float L = 0.0f;
-        for (int sp = s8; sp < nsp32; sp += 8) {
-            float w = 0.0f;
-            if (sp < P.nsplit) {
-                w = __builtin_amdgcn_exp2f(tM[sp * kMaxGroupHeads + hh] - Mu);
-                L += w * tL[sp * kMaxGroupHeads + hh];
-            }
-            sW[hh * nsp32 + sp] = w;
-        }
-        L = head_sum(L);
-        if (s8 == 0) {
-            sHead[hh] = M;
-            sHead[kMaxGroupHeads + hh] = L;
-        }
-        PROF(13);
+        if (appends) step_end<BITS, GS, BF16>(lds, bi, hk, step_len);
     }
-    __syncthreads();
-    PROF(14);
-    for (int idx = tid; idx < g * kHeadDim; idx += NW * 64) {
-        const int hh = idx >> 7, c = idx & 127;
-        const int hq = hk * g + hh;
-        float O = 0.0f;
-        for (int s0 = 0; s0 < P.nsplit; s0 += 32) {
-            if (idx != tid || s0 != 0) {
-                load_partials(v0, o_part, static_cast<uint32_t>((row00 + hh) * kHeadDim + c), hstride * kHeadDim, s0,
-                              P.nsplit);
-            }
-#pragma unroll
-            for (int k = 0; k < 32; k += 4) {
-                const f4 w4 = *reinterpret_cast<const f4*>(&sW[hh * nsp32 + s0 + k]);
-                O += w4[0] * v0[k];
-                O += w4[1] * v0[k + 1];
-                O += w4[2] * v0[k + 2];
-                O += w4[3] * v0[k + 3];
-            }
-        }
-        const float M = sHead[hh], L = sHead[kMaxGroupHeads + hh];
-        const bool none = !(L > 0.0f);
-        out[bi * out_sb + hq * out_sh + c] = to_out<BF16>(none ? 0.0f : O / L);
-        if (c == 0 && lse_out) {
-            lse_out[row00 + hh] = none ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
-        }
-    }
-    }   // nsplit > 1
-    // here: the workgroup that wrote the output of its (batch, kv-head)
-    if constexpr (APPEND) step_end<BITS, GS, BF16>(lds, bi, hk, step_len);
     PROF(7);
     PROF_FLUSH();
 }

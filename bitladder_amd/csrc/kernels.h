@@ -5,6 +5,11 @@
 
 namespace bitdecode {
 
+// Arrival counters of different query heads are drawn from compute units all over the chip at about the
+// same time: each sits in a 256-byte block of its own (counters that share a cache line cost several
+// microseconds per launch on a multi-die GPU, measured).
+constexpr int kTicketStride = 64;      // ints
+
 struct QpackParams {
     const uint16_t* k;
     const uint16_t* v;
@@ -40,8 +45,8 @@ struct FwdParams {
     const int* reslens;
     int seqlen, reslen;
     float* o_part;      // [split][b][h][128] partial outputs, relative to the split's own maximum
-    float* ml_part;     // [split][b][h][2] maximum (base-2 units) and sum of each split
-    int* tickets;       // [b][h_k] arrival counters, zero between calls
+    float* ml_part;     // [b][h][split][2] maximum (base-2 units) and sum of each split
+    int* tickets;       // [b][h] arrival counters, kTicketStride ints apart, zero between calls
     uint16_t* out;
     int64_t out_sb, out_sh;
     float* lse;         // optional [b][h]
@@ -58,7 +63,7 @@ struct FwdParams {
     // window's next row, stored there, and a window that becomes full is packed behind the prefix.
     // seqlens / reslens / seqlen / reslen are not used then.
     int* lengths;               // [b], advanced by one by the last workgroup of each sequence
-    int* step_tickets;          // [b] arrival counters, zero between calls
+    int* step_tickets;          // [b] arrival counters, kTicketStride ints apart, zero between calls
     const uint16_t* k_new;
     const uint16_t* v_new;
     int64_t knew_sb, knew_sh, vnew_sb, vnew_sh;

@@ -92,9 +92,11 @@ typedef struct bitdecode_fwd_args {
     int64_t out_stride_b, out_stride_h;
     float* softmax_lse;        /* optional [b, h] natural-log LSE                           */
     void* workspace;           /* >= bitdecode_fwd_workspace_bytes(...) or NULL if 1 split;
-                                  its first 4*b*h bytes (arrival counters) must be zero before
-                                  the first call and are left zero by every call; calls that
-                                  share a workspace must not overlap in time                */
+                                  ordinary device memory (hipMalloc); its first 256*b*h bytes
+                                  (one arrival counter per query head, each in a 256-byte block
+                                  of its own) must be zero before the first call and are left
+                                  zero by every call; calls that share a workspace must not
+                                  overlap in time                                            */
     size_t workspace_bytes;
     int32_t b, h, h_k, d;      /* d must be 128, h % h_k == 0, h / h_k <= 8                 */
     int32_t bits, group_size, dtype;
