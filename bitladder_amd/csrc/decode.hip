@@ -44,6 +44,10 @@
 #include "layout.h"
 #include "qpack_chunk.h"
 
+#ifndef X_DEPTH
+#define X_DEPTH 4
+#endif
+
 namespace bitdecode {
 namespace {
 
@@ -333,6 +337,7 @@ struct UnitCfg {
     static constexpr int OFF_KP = 8192, OFF_VP = 8192 + 2 * KPB;
     static constexpr int REGION = unit_region_bytes(BITS, GS);
     static constexpr int NW = decode_waves(BITS, GS);        // waves per workgroup
+    static constexpr int DEPTH = (X_DEPTH) < NKP + RPS + 1 ? (X_DEPTH) : NKP + RPS + 1;   // rows a wave keeps in flight
     static_assert(REGION == OFF_VP + VPB && REGION % 256 == 0, "region layout");
     static_assert(NW % 4 == 0, "the merge reads four wave weights per LDS access");
 };
@@ -347,7 +352,7 @@ __device__ __forceinline__ void dma_row(const uint8_t* base, uint32_t lane16, ui
     static_assert(OFFSET >= 0 && OFFSET < 4096, "immediate offset field");
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
                  :
-                 : "v"(lane16), "s"(base), "s"(lds_base), "n"(OFFSET)
+                 : "v"(lane16), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_base)), "n"(OFFSET)
                  : "memory", "m0");
 }
 
@@ -365,7 +370,7 @@ __device__ __forceinline__ void dma_row_first_lanes(const uint8_t* base, uint32_
                  "global_load_lds_dwordx4 %1, %2 offset:%4\n\t"
                  "s_mov_b64 exec, %0"
                  : "=&s"(saved)
-                 : "v"(lane16), "s"(base), "s"(lds_base), "n"(OFFSET), "s"(mask)
+                 : "v"(lane16), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_base)), "n"(OFFSET), "s"(mask)
                  : "memory", "m0", "scc");
 }
 
@@ -489,23 +494,108 @@ __device__ __forceinline__ void dma_bytes(const uint8_t* src, uint32_t lane16, u
         dma_bytes<BYTES, R + 1>(src, lane16, lds_dst);
     }
 }
+// ---- the rows of a unit as a pipeline
+// A compute unit returns loads in the order it issued them, accepts only about 64 KB of them at a time,
+// and while a wave's load waits to be accepted no other wave of that SIMD gets an LDS instruction
+// through (measured: LDS reads of all waves stall for as long as load instructions queue up).  So a wave
+// never sends a whole unit at once.  The rows of a unit are numbered in the order they are consumed:
+//   K parameters | per 64-token step: its K rows, (first step: V parameters,) its V rows
+// and a wave keeps kDepth of them in flight: the prologue issues rows 0 .. kDepth-2 of the wave's first
+// unit, and just before the wave waits for row i it issues row i + kDepth - 1 (running on into the next
+// unit of the wave).  With all waves of a workgroup doing this the rows of different waves interleave in
+// the memory queue, the waves finish together, and what is left after the last byte of the stream is the
+// work on one row per wave.  Before row i is read exactly kDepth - 1 younger loads may still be in flight
+// (fewer at the end of the wave's last unit), which is what the s_waitcnt in front of every read says.
+
+struct RowId {
+    int kind;      // 0 K parameters, 1 K codes, 2 V parameters, 3 V codes
+    int idx;       // 1 KB row inside its kind
+};
 template <int BITS, int GS>
-__device__ __forceinline__ void issue_kside(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region, int kslot) {
+constexpr RowId row_at(int i) {
     using C = UnitCfg<BITS, GS>;
-    dma_bytes<C::KPB>(A.kp, lane16, region + C::OFF_KP + kslot * C::KPB);
-    dma_row<0>(A.kc, lane16, region);
-    dma_row<1024>(A.kc, lane16, region);
-    dma_row<2048>(A.kc, lane16, region);
-    dma_row<3072>(A.kc, lane16, region);
+    if (i < C::NKP) return RowId{0, i};
+    int p = i - C::NKP;
+    for (int s = 0; s < C::NSTEP; ++s) {
+        if (p < C::RPS) return RowId{1, s * C::RPS + p};
+        p -= C::RPS;
+        if (s == 0) {
+            if (p < C::NVP) return RowId{2, p};
+            p -= C::NVP;
+        }
+        if (p < C::RPS) return RowId{3, s * C::RPS + p};
+        p -= C::RPS;
+    }
+    return RowId{-1, 0};
 }
+// position of a row in that order
 template <int BITS, int GS>
-__device__ __forceinline__ void issue_vside(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region) {
+constexpr int pos_of(int kind, int idx) {
     using C = UnitCfg<BITS, GS>;
-    dma_bytes<C::VPB>(A.vp, lane16, region + C::OFF_VP);
-    dma_row<0>(A.vc, lane16, region + 4096);
-    dma_row<1024>(A.vc, lane16, region + 4096);
-    dma_row<2048>(A.vc, lane16, region + 4096);
-    dma_row<3072>(A.vc, lane16, region + 4096);
+    for (int i = 0; i < C::KSIDE + C::VSIDE; ++i) {
+        const RowId r = row_at<BITS, GS>(i);
+        if (r.kind == kind && r.idx == idx) return i;
+    }
+    return -1;
+}
+// the load of row I of a unit into the wave's region; kslot names the K-parameter slot of that unit
+template <int BITS, int GS, int I>
+__device__ __forceinline__ void issue_row(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region, int kslot) {
+    using C = UnitCfg<BITS, GS>;
+    constexpr RowId r = row_at<BITS, GS>(I);
+    static_assert(r.kind >= 0, "row inside the unit");
+    if constexpr (r.kind == 0) {
+        constexpr int left = C::KPB - r.idx * 1024;
+        const uint32_t dst = region + C::OFF_KP + kslot * C::KPB;
+        if constexpr (left >= 1024) {
+            dma_row<r.idx * 1024>(A.kp, lane16, dst);
+        } else {
+            dma_row_first_lanes<r.idx * 1024, left / 16>(A.kp, lane16, dst);
+        }
+    } else if constexpr (r.kind == 1) {
+        dma_row<r.idx * 1024>(A.kc, lane16, region);
+    } else if constexpr (r.kind == 2) {
+        constexpr int left = C::VPB - r.idx * 1024;
+        if constexpr (left >= 1024) {
+            dma_row<r.idx * 1024>(A.vp, lane16, region + C::OFF_VP);
+        } else {
+            dma_row_first_lanes<r.idx * 1024, left / 16>(A.vp, lane16, region + C::OFF_VP);
+        }
+    } else {
+        dma_row<r.idx * 1024>(A.vc, lane16, region + 4096);
+    }
+}
+// prologue of a wave: rows 0 .. kDepth-2 of its first unit
+template <int BITS, int GS, int I = 0>
+__device__ __forceinline__ void issue_first_rows(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region) {
+    if constexpr (I < UnitCfg<BITS, GS>::DEPTH - 1) {
+        issue_row<BITS, GS, I>(A, lane16, region, 0);
+        issue_first_rows<BITS, GS, I + 1>(A, lane16, region);
+    }
+}
+// In front of the read of row I of the current unit: send the row that keeps the pipeline full (of this
+// unit, or of the next one if there is one), then wait until row I has landed.  The load may overwrite
+// rows read earlier: every LDS read issued so far has to have returned its data first (a read that has
+// only been issued can be overtaken by the load's write).
+template <int BITS, int GS, bool HAS_NEXT, int I>
+__device__ __forceinline__ void row_ready(const UnitAddr<BITS, GS>& cur, const UnitAddr<BITS, GS>& next, uint32_t lane16,
+                                          uint32_t region, int kslot) {
+    using C = UnitCfg<BITS, GS>;
+    constexpr int ROWS = C::KSIDE + C::VSIDE, kDepth = C::DEPTH, J = I + kDepth - 1;
+    // rows of the next unit fetched from inside this one land on K-side rows only: the V parameters of this
+    // unit are still in use up to its last row
+    static_assert(kDepth - 1 <= C::NKP + C::RPS && kDepth - 1 < ROWS, "depth of the row pipeline");
+    if constexpr (J < ROWS) {
+        wait_lds_reads();
+        issue_row<BITS, GS, J>(cur, lane16, region, kslot);
+        wait_vm<kDepth - 1>();
+    } else if constexpr (HAS_NEXT) {
+        wait_lds_reads();
+        issue_row<BITS, GS, J - ROWS>(next, lane16, region, kslot ^ 1);
+        wait_vm<kDepth - 1>();
+    } else {
+        wait_vm<ROWS - 1 - I>();
+    }
 }
 
 // Per-group state of the K side: Q with the group's scale folded in (exact hi/lo split) and the
@@ -559,18 +649,19 @@ __device__ __forceinline__ void start_group(KGroup& G, const uint8_t* kpar, cons
 
 // One packed unit from the wave's LDS region, in 64-token steps: S^T tiles of the step, online
 // softmax update, O^T += V^T P^T for the same tokens.  Scores stay in q.k units; the softmax
-// scale is applied inside the exponent.  On entry both sides of the unit are in flight or landed
-// (queue order: K side, V side).  With HAS_NEXT the two sides of the wave's next unit are issued
-// from here (see above); kslot says which K-parameter slot the current unit uses.
-template <int BITS, int GS, bool BF16, bool HAS_NEXT, bool DEFER_V = false>
+// scale is applied inside the exponent.  On entry rows 0 .. kDepth-2 of the unit are in flight or landed;
+// with HAS_NEXT the first rows of the wave's next unit are issued from here (see above); kslot says
+// which K-parameter slot the current unit uses.
+template <int BITS, int GS, bool BF16, bool HAS_NEXT>
 __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, int kslot,
-                                             const UnitAddr<BITS, GS>& next, const QRows& Q, const FwdParams& P,
-                                             int lane, bool lo_part, const Magic& mg, WaveState<kHeadDim / GS>& st,
-                                             unsigned long long* phase_ts = nullptr) {
+                                             const UnitAddr<BITS, GS>& cur, const UnitAddr<BITS, GS>& next,
+                                             const QRows& Q, const FwdParams& P, int lane, bool lo_part, const Magic& mg,
+                                             WaveState<kHeadDim / GS>& st) {
     using C = UnitCfg<BITS, GS>;
     constexpr int NCG = C::NCG, TPS = C::TPS, NKS = C::NKS, TPG = C::TPG, CTPG = GS / 16;
-    constexpr int NSTEP = C::NSTEP, RPS = C::RPS;
+    constexpr int NSTEP = C::NSTEP, RPS = C::RPS, TPR = TPS / RPS;      // tiles per K row
     const int kg = lane >> 4;
+    const uint32_t lane16 = lane * 16;
     const h8 noff = -code_offsets<BITS>();
     const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
     const uint32_t hi_cols = lo_part ? 0u : 0xffffffffu;
@@ -578,26 +669,30 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     const u4* vcode = reinterpret_cast<const u4*>(reg + 4096) + lane;
     const uint8_t* kpar = reg + C::OFF_KP + kslot * C::KPB;
     const uint8_t* vpar = reg + C::OFF_VP + kg * 16;
+#define ROW_READY(kind, idx) row_ready<BITS, GS, HAS_NEXT, pos_of<BITS, GS>(kind, idx)>(cur, next, lane16, region_lds, kslot)
 
-    static_assert(!(HAS_NEXT && DEFER_V), "only a wave's single unit defers its V side");
     // the K parameters lead the queue: the first K group is prepared while the code rows arrive
-    constexpr int VQ0 = DEFER_V ? 0 : C::VSIDE;      // V-side loads behind the K side while step 0 runs
-    wait_vm<4 + VQ0>();
-    PHASE(8);
+#pragma unroll
+    for (int i = 0; i < C::NKP; ++i) {
+        if (i == 0) ROW_READY(0, 0);
+        if (i == 1) ROW_READY(0, 1);
+    }
+    static_assert(C::NKP <= 2 && C::NVP <= 2, "parameter rows of a unit");
     KGroup G;
     start_group<BITS, BF16>(G, kpar, Q, kg);
-    (void)phase_ts;
 #pragma unroll
     for (int step = 0; step < NSTEP; ++step) {
-        constexpr int kLast = NSTEP - 1;
-        // still allowed in flight: the K rows of later steps and the whole V side
-        wait_vm<4 - RPS + VQ0>();
-        if (step > 0) wait_vm<C::VSIDE>();
-        PHASE(9 + 3 * step);
         f4 sc[TPS];
 #pragma unroll
         for (int tt = 0; tt < TPS; ++tt) {
             const int tile = step * TPS + tt;
+            if (tt % TPR == 0) {       // the K row of this tile (4 bits: one tile per row, 2 bits: two)
+                const int row = tile / TPR;
+                if (row == 0) ROW_READY(1, 0);
+                if (row == 1) ROW_READY(1, 1);
+                if (row == 2) ROW_READY(1, 2);
+                if (row == 3) ROW_READY(1, 3);
+            }
             if (tile != 0 && tile % TPG == 0) {
                 start_group<BITS, BF16>(G, kpar + ((tile * 16) / GS) * kKParamGroupBytes, Q, kg);
             }
@@ -618,12 +713,6 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
             }
             sc[tt] = acc;
         }
-        // every K row and this unit's K parameters have been read: the next unit's K side may land
-        if (HAS_NEXT && step == kLast) {
-            wait_lds_reads();
-            issue_kside<BITS, GS>(next, lane * 16, region_lds, kslot ^ 1);
-        }
-        PHASE(10 + 3 * step);
 
         static_assert(TPS == 4 && NKS == 2, "four tiles, two sub-blocks per step");
         h8 p16[NKS], pz[NKS], pm[NKS];
@@ -634,24 +723,14 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
         }
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) st.l = mfma32(ones, pz[ks], st.l);
-        if (DEFER_V && step == 0) {
-#ifdef X_PRIO
-            __builtin_amdgcn_s_setprio(0);
-#endif
-            issue_vside<BITS, GS>(next, lane * 16, region_lds);      // `next` is this unit here
-        }
-        PHASE(11 + 3 * step);
-        // V side of the step, row by row in the order the rows arrive.  A row holds one channel half
-        // (tiles ct = 4*hf .. 4*hf+3) of one 32-token sub-block (4 bits) or of the whole step (2 bits).
-        // Still allowed in flight behind row r of the unit: the rows after it and, once issued, the
-        // next unit's K side.  A wave's last unit waits row by row, so that only the products of the
-        // last row are left when the last byte lands; a unit with a successor waits once per step.
-        constexpr int kNextK = HAS_NEXT ? C::KSIDE : 0;
-        const int behind = (step == kLast) ? kNextK : 0;
-        if constexpr (HAS_NEXT) {
-            wait_vm_n(behind + 4 - (step + 1) * RPS);
-        } else if (step == 0) {
-            wait_vm<4>();              // the V parameters
+        // V side of the step, row by row.  A row holds one channel half (tiles ct = 4*hf .. 4*hf+3) of one
+        // 32-token sub-block (4 bits) or of the whole step (2 bits).
+        if (step == 0) {
+#pragma unroll
+            for (int i = 0; i < C::NVP; ++i) {
+                if (i == 0) ROW_READY(2, 0);
+                if (i == 1) ROW_READY(2, 1);
+            }
         }
         h8 pp[NCG][NKS];
         constexpr int CGH = NCG >= 2 ? NCG / 2 : 1;      // channel groups per channel half
@@ -675,8 +754,12 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
                     }
                 }
             }
-            if constexpr (!HAS_NEXT) wait_vm_n(3 - (step * RPS + r));
-            const u4 w = vcode[64 * (step * RPS + r)];
+            const int vrow = step * RPS + r;
+            if (vrow == 0) ROW_READY(3, 0);
+            if (vrow == 1) ROW_READY(3, 1);
+            if (vrow == 2) ROW_READY(3, 2);
+            if (vrow == 3) ROW_READY(3, 3);
+            const u4 w = vcode[64 * vrow];
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
                 const int ct = 4 * hf + x, cg = ct / CTPG;
@@ -691,12 +774,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
             }
         }
     }
-    // every V row and the V parameters have been read: the next unit's V side may land
-    if (HAS_NEXT) {
-        wait_lds_reads();
-        issue_vside<BITS, GS>(next, lane * 16, region_lds);
-    }
-    PHASE(15);
+#undef ROW_READY
 }
 
 // Fields of the kernel's parameter block, re-read from the kernarg segment at the point of use.  The
@@ -1159,29 +1237,11 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         qa_raw = load_untracked(q0 + (hq < g ? hq : 0) * P.q_sh);
         qb_raw = load_untracked(q0 + (hq + 4 < g ? hq + 4 : 0) * P.q_sh);
     }
-    // First units: every wave of the workgroup sends out its K side before any wave sends its V side
-    // (loads come back roughly in the order the compute unit issued them).  The K sides then land in
-    // the first half of the stream and the scores and probabilities of all waves are ready while the V
-    // sides are still arriving: after the last byte only the products of the last V row are left.
-    // (A bare s_barrier: no wait for the loads in flight.)
     UnitAddr<BITS, GS> A;
-#ifdef X_DEFERV
-    const bool single = u + NW >= u1;      // at most one packed unit for this wave
-#else
-    const bool single = false;
-#endif
     if (u < u1) {
-#ifdef X_PRIO
-        __builtin_amdgcn_s_setprio(3);
-#endif
         A = unit_addr<BITS, GS>(P, bi, hk, u);
-        issue_kside<BITS, GS>(A, lane * 16, region_lds, 0);
-        if (!single) {
-            issue_vside<BITS, GS>(A, lane * 16, region_lds);
-            wait_then_take<C::KSIDE + C::VSIDE>(qa, qb, qa_raw, qb_raw);
-        } else {
-            wait_then_take<C::KSIDE>(qa, qb, qa_raw, qb_raw);
-        }
+        issue_first_rows<BITS, GS>(A, lane * 16, region_lds);
+        wait_then_take<C::DEPTH - 1>(qa, qb, qa_raw, qb_raw);
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
     }
@@ -1214,24 +1274,17 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     if (u < u1) {
         const Magic mg;
 #ifdef BITDECODE_PROF
-        if (single) wait_vm<4>(); else wait_vm<4 + C::VSIDE>();   // K parameters have arrived
+        wait_vm<C::DEPTH - 2>();   // first row (K parameters) has arrived
         PROF(2);
-        unsigned long long* phase_ts = prof_ts;
-#else
-        unsigned long long* phase_ts = nullptr;
 #endif
         int kslot = 0;
         for (int un = u + NW; un < u1; un += NW) {        // units that have a successor: it is fetched from inside
-            A = unit_addr<BITS, GS>(P, bi, hk, un);
-            compute_unit<BITS, GS, BF16, true>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
+            const UnitAddr<BITS, GS> An = unit_addr<BITS, GS>(P, bi, hk, un);
+            compute_unit<BITS, GS, BF16, true>(region, region_lds, kslot, A, An, Q, P, lane, lo_part, mg, st);
+            A = An;
             kslot ^= 1;
-            phase_ts = nullptr;
         }
-        if (single) {     // (the wave's only unit: its V side is still to be issued)
-            compute_unit<BITS, GS, BF16, false, true>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
-        } else {
-            compute_unit<BITS, GS, BF16, false>(region, region_lds, kslot, A, Q, P, lane, lo_part, mg, st, phase_ts);
-        }
+        compute_unit<BITS, GS, BF16, false>(region, region_lds, kslot, A, A, Q, P, lane, lo_part, mg, st);
     }
     PROF(3);
     // ---- fp16 window tiles of this wave (the region becomes the V-transpose slab)
