@@ -223,6 +223,8 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
     if (nsplit > 512) return fail(BITDECODE_EINVAL, "num_splits %d is above the limit of 512", nsplit);
     if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
+    if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim * sizeof(float) >= (size_t(1) << 31))
+        return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d heads: partial outputs of 2 GiB or more", nsplit, a->b, a->h);
     if (nsplit > 1 || step) {
         const size_t need = step ? bitdecode_fwd_append_workspace_bytes(a->b, a->h, nsplit)
                                  : bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);

@@ -171,7 +171,7 @@ __device__ __forceinline__ f4 mfma16(h4 a, h4 b, f4 c) {
 
 // value held by the partner column (lane ^ 8 inside each row of 16 lanes): DPP row_ror:8
 __device__ __forceinline__ float partner(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, true));
 }
 // (every lane has a source lane, so the "bound control" flag changes nothing but tells the compiler
 // that no previous value of the result survives, which saves it a move)
@@ -975,71 +975,69 @@ __device__ __forceinline__ float row_sum16(float x) {
     x += row_ror<2>(x);
     return x + row_ror<1>(x);
 }
-// the same over the whole wave, as a scalar
+// the maximum over the whole wave, as a scalar
 __device__ __forceinline__ float wave_max(float x) {
     x = row_max16(x);
     return fmaxf(fmaxf(lane_value(x, 0), lane_value(x, 16)), fmaxf(lane_value(x, 32), lane_value(x, 48)));
 }
-__device__ __forceinline__ float wave_sum(float x) {
-    x = row_sum16(x);
-    return (lane_value(x, 0) + lane_value(x, 16)) + (lane_value(x, 32) + lane_value(x, 48));
-}
 
-// partial outputs (two channels per lane) of splits s0 .. s0+31, clamped to the last split
-__device__ __forceinline__ void load_partials(float2 (&v)[32], const float* base, int64_t split_stride, int s0, int nsplit) {
-    base += static_cast<int64_t>(s0) * split_stride;
-    const int cnt = min(32, nsplit - s0);
+// 8 bytes per lane at (wave-uniform base) + (32-bit lane offset): the base stays in scalar registers, so a
+// run of such loads costs two scalar additions per load and no vector address arithmetic
+__device__ __forceinline__ float2 ld_dev2_at(const float* base, uint32_t lane_bytes) {
+    return ld_dev2(reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes));
+}
+// partial outputs (two channels per lane) of splits s0 .. s0+31 of one query head; past the last split the
+// last one is read again (its weight is zero)
+__device__ __forceinline__ void load_partials(float2 (&v)[32], const float* head_base, uint32_t lane_bytes,
+                                              uint32_t split_stride, int s0, int nsplit) {
+    const float* base = head_base + static_cast<size_t>(s0) * split_stride;
+    const int cnt = nsplit - s0;
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
-        v[k] = ld_dev2(base);
-        if (k + 1 < cnt) base += split_stride;
+        v[k] = ld_dev2_at(base, lane_bytes);
+        base += (k + 1 < cnt) ? split_stride : 0u;
     }
 }
 
 // Merge of the splits of one query head by one wave (flash_fwd_kernel.h:1217-1298 in unnormalised
 // form): out = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M).  Lane l owns channels 2l and
-// 2l+1; the (M, L) pairs are spread over the lanes (split s0 + l of each round of 64), the weights go
-// back to all lanes as scalars.  The order of the additions is fixed.
-__device__ __forceinline__ void merge_splits(const float* o_part, const float* ml_part, int64_t hrow, int64_t hstride,
+// 2l+1.  Splits are taken 32 at a time: lane l holds the (M, L) pair of split s0 + l % 32, the weights go
+// back to all lanes as scalars.  The order of the additions is fixed.  `split_stride` is in floats and,
+// like the whole partial-output area, below 2^31 bytes (checked by the host).
+__device__ __forceinline__ void merge_splits(const float* o_part, const float* ml_part, int64_t hrow, uint32_t split_stride,
                                              int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
-    const float* ob = o_part + hrow * kHeadDim + 2 * lane;
-    const int64_t sstride = hstride * kHeadDim;
+    const float* head_base = o_part + hrow * kHeadDim;
     const float* mlb = ml_part + hrow * nsplit * 2;
+    const uint32_t lane_bytes = lane * 8, ml_lane = (lane & 31) * 8;
+    const int sl = lane & 31;
     const float2 none = float2{-INFINITY, 0.0f};
-    const float2 ml0 = lane < nsplit ? ld_dev2(mlb + 2 * lane) : none;      // ahead of the bulk loads
     float2 v[32];
-    load_partials(v, ob, sstride, 0, nsplit);
-    float mx = ml0.x;
-    for (int sb = 64; sb < nsplit; sb += 64) {
-        if (sb + lane < nsplit) mx = fmaxf(mx, ld_dev2(mlb + 2 * (sb + lane)).x);
-    }
-    M = wave_max(mx);
-    const float Mu = (M == -INFINITY) ? 0.0f : M;
-    float lacc = 0.0f;
+    float2 ml = none;
+    float lacc = 0.0f, Mu = 0.0f;
     O0 = O1 = 0.0f;
-    for (int sb = 0; sb < nsplit; sb += 64) {
-        float2 ml = ml0;
-        if (sb > 0) ml = sb + lane < nsplit ? ld_dev2(mlb + 2 * (sb + lane)) : none;
-        const float w = __builtin_amdgcn_exp2f(ml.x - Mu);       // 0 past the last split
+    for (int s0 = 0; s0 < nsplit; s0 += 32) {
+        if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
+        load_partials(v, head_base, lane_bytes, split_stride, s0, nsplit);
+        if (s0 == 0) {
+            float mx = ml.x;
+            for (int s = 32; s < nsplit; s += 32) {        // more than 32 splits: the other maxima
+                if (s + sl < nsplit) mx = fmaxf(mx, ld_dev2_at(mlb + 2 * s, ml_lane).x);
+            }
+            M = wave_max(mx);
+            Mu = (M == -INFINITY) ? 0.0f : M;
+        }
+        const float w = (s0 + sl < nsplit) ? __builtin_amdgcn_exp2f(ml.x - Mu) : 0.0f;
         lacc = __builtin_fmaf(w, ml.y, lacc);
-        if (sb > 0) load_partials(v, ob, sstride, sb, nsplit);
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             const float wk = lane_value(w, k);
             O0 = __builtin_fmaf(wk, v[k].x, O0);
             O1 = __builtin_fmaf(wk, v[k].y, O1);
         }
-        if (sb + 32 < nsplit) {
-            load_partials(v, ob, sstride, sb + 32, nsplit);
-#pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                const float wk = lane_value(w, 32 + k);
-                O0 = __builtin_fmaf(wk, v[k].x, O0);
-                O1 = __builtin_fmaf(wk, v[k].y, O1);
-            }
-        }
     }
-    L = wave_sum(lacc);
+    // both halves of the wave hold the same 32 terms
+    const float lrow = row_sum16(lacc);
+    L = lane_value(lrow, 0) + lane_value(lrow, 16);
 }
 
 template <bool BF16>
@@ -1411,7 +1409,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
             if constexpr (APPEND) {
                 if (wave == 0) *s_last = last;
             } else if (last) {
-                merge_splits(o_part, ml_part, hrow, hstride, P.nsplit, lane, O0, O1, M, L);
+                merge_splits(o_part, ml_part, hrow, static_cast<uint32_t>(hstride) * kHeadDim, P.nsplit, lane, O0, O1, M, L);
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
             }
         }
@@ -1426,7 +1424,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
             appends = *s_last != 0;
             if (appends) step_begin<NW>(bi, hk, step_len);
             if (wave < g && last) {
-                merge_splits(o_part, ml_part, hrow, hstride, P.nsplit, lane, O0, O1, M, L);
+                merge_splits(o_part, ml_part, hrow, static_cast<uint32_t>(hstride) * kHeadDim, P.nsplit, lane, O0, O1, M, L);
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
             }
         }
