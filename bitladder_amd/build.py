@@ -24,6 +24,7 @@ PER_FILE = {
     "qpack.hip": ["-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"],
     "decode.hip": ["-mllvm", "-amdgpu-sched-strategy=gcn-max-ilp", "-fhip-fp32-correctly-rounded-divide-sqrt"],
     "api.hip": [],
+    "probe.hip": [],
 }
 
 

@@ -141,7 +141,8 @@ class BitKVCache:
             k_new, v_new = k_new[:, None], v_new[:, None]
         if any(p + r + 1 > self.capacity for p, r in zip(self.packed_len, self.res_len)):
             raise ValueError("step: cache capacity exceeded")
-        plan = self.plan_step(q, k_new.to(self.dtype), v_new.to(self.dtype), softmax_scale, **kw)
+        # (the step's workspace comes from the per-stream cache: nothing is allocated or filled per token)
+        plan = self.plan_step(q, k_new.to(self.dtype), v_new.to(self.dtype), softmax_scale, _stream_ws=True, **kw)
         with torch.cuda.device(self.device):
             out = plan.run()
         for i, (p, r) in enumerate(zip(self.packed_len, self.res_len)):

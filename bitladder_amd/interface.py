@@ -91,6 +91,26 @@ def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+# Split workspaces of the plain entry points, one per (device, stream, kind, batch, heads, splits): a call
+# leaves the arrival counters at the head of its workspace at zero, so the next call on the same stream can
+# take the same buffer without refilling it (calls on one stream run one after the other; two streams never
+# share a buffer).  Plans own their workspace instead: they may be replayed from anywhere.
+_WORKSPACES: "dict[tuple, torch.Tensor]" = {}
+_MAX_WORKSPACES = 64
+
+
+def _stream_workspace(device, kind: str, b: int, h: int, ns: int, nbytes: int) -> torch.Tensor:
+    key = (device.index, _stream_ptr(device), kind, b, h, ns)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        if len(_WORKSPACES) >= _MAX_WORKSPACES:
+            _WORKSPACES.pop(next(iter(_WORKSPACES)))
+        # zero-filled once: the arrival counters must be 0 before the first call
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
 def _i32_dev(x, b, device, name):
     if not isinstance(x, torch.Tensor):
         raise TypeError(f"{name} must be a tensor")
@@ -205,7 +225,8 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
                          max_residual_len: Optional[int] = None,
                          num_splits: int = 0,
                          out: Optional[torch.Tensor] = None,
-                         return_lse: bool = False) -> DecodePlan:
+                         return_lse: bool = False,
+                         _stream_ws: bool = False) -> DecodePlan:
     """Validates a decode call and returns a `DecodePlan`; see `fwd_kvcache_int`."""
     _check_quant(quant_mode, group_size, num_bits)
     if q.dim() != 4 or q.shape[1] != 1:
@@ -302,7 +323,8 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
         if nbytes:
             # zero-filled: the arrival counters at its head must be 0 before the first call
             # (every call leaves them at 0 again)
-            ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+            ws = (_stream_workspace(device, "fwd", b, h, ns, nbytes) if _stream_ws
+                  else torch.zeros(nbytes, dtype=torch.uint8, device=device))
             keep.append(ws)
             a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
     return DecodePlan(a, out, lse, tuple(keep), device)
@@ -332,8 +354,10 @@ def fwd_kvcache_int(q: torch.Tensor,
       num_splits        0 = choose; out = preallocated output; return_lse -> (out, lse [b, h])
     """
     return_lse = kwargs.get("return_lse", False)
+    # the split workspace comes from a per-stream cache: no allocation and no fill after the first call
+    # (the reference allocates its accumulators per call, decode_api.cpp:292-295, 375-390)
     plan = plan_fwd_kvcache_int(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale,
-                                quant_mode, group_size, num_bits, **kwargs)
+                                quant_mode, group_size, num_bits, _stream_ws=True, **kwargs)
     with torch.cuda.device(plan.device):
         plan.run()
     return (plan.out, plan.lse) if return_lse else plan.out
@@ -352,7 +376,8 @@ def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: tor
                                 *,
                                 num_splits: int = 0,
                                 out: Optional[torch.Tensor] = None,
-                                return_lse: bool = False) -> DecodePlan:
+                                return_lse: bool = False,
+                                _stream_ws: bool = False) -> DecodePlan:
     """Validates a decode step with append and returns its `DecodePlan`; see `fwd_kvcache_int_append`."""
     if k_residual is None or v_residual is None or k_residual.dim() != 4 or k_residual.shape[1] < CHUNK:
         raise RuntimeError(f"the residual window must hold at least {CHUNK} tokens")
@@ -385,7 +410,8 @@ def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: tor
         a.fwd.num_splits = ns
         nbytes = L.bitdecode_fwd_append_workspace_bytes(b, h, ns)
         # zero-filled: the arrival counters must be 0 before the first call (every call leaves them at 0)
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        ws = (_stream_workspace(device, "step", b, h, ns, nbytes) if _stream_ws
+              else torch.zeros(nbytes, dtype=torch.uint8, device=device))
         a.fwd.workspace, a.fwd.workspace_bytes = ws.data_ptr(), nbytes
     keep = inner._keep + (k_new, v_new, lengths, ws)
     return DecodePlan(a, inner.out, inner.lse, keep, device)
@@ -415,7 +441,7 @@ def fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Te
     return_lse = kwargs.get("return_lse", False)
     plan = plan_fwd_kvcache_int_append(q, k_new, v_new, k_pack, k_params, v_pack, v_params, k_residual, v_residual,
                                        lengths, max_len, opt_block_table, softmax_scale, quant_mode, group_size,
-                                       num_bits, **kwargs)
+                                       num_bits, _stream_ws=True, **kwargs)
     with torch.cuda.device(plan.device):
         plan.run()
     return (plan.out, plan.lse) if return_lse else plan.out

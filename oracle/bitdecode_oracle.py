@@ -9,7 +9,7 @@ Every function cites the reference code it follows (paths relative to the refere
 tree).  The reference cannot be compiled here (CUDA/PTX only, CUTLASS submodule
 absent), so each function is pinned by closed forms, invariants, brute force and a
 second, independently written C restatement (oracle/bitdecode_oracle.c); the tests
-that do so live in tests/test_oracle_*.py.
+that do so live in tests/test_oracle.py.
 
 Pin status
 ----------
@@ -20,7 +20,8 @@ quantize_group / quantize_kv_ref : pinned (closed forms, invariants, brute-force
     binary's `scale` on rare groups are "parity unpinned".  So is the sign of a
     stored zero-point that is a zero of a group holding both -0 and +0: the reference
     reduces with `x < y ? x : y`, order-dependent; here -0 orders below +0.
-dequantize_ref  : pinned (exact small-integer arithmetic).
+dequantize_ref  : pinned (exactness on an exact grid, error bound scale/2 against the input, one-hot
+    probes of the K and V grouping axes; tests/test_oracle.py).
 attend_ref      : pinned (reduces to softmax(QK^T)V; block-order invariance).
 lse_combine_ref : pinned (closed form, split-count invariance).
 num_splits_heuristic_ref : pinned (known answers from the reference's own comment).

@@ -79,3 +79,14 @@ def assert_cache_equals_oracle(cache_np, qkv: O.QuantKV):
     np.testing.assert_array_equal(kz, stored(qkv.k_zero), err_msg="K zero")
     np.testing.assert_array_equal(vs, stored(qkv.v_scale), err_msg="V scale")
     np.testing.assert_array_equal(vz, stored(qkv.v_zero), err_msg="V zero")
+
+
+def out_tolerance(want: np.ndarray, dtype: str, atol: float = 2e-3) -> np.ndarray:
+    """Element-wise bound on |output - oracle|: 2e-3 for the arithmetic, plus, for a bf16 output, half a
+    bf16 unit in the last place of the expected value (what rounding the result to 8 significant bits adds)."""
+    want = np.asarray(want, dtype=np.float32)
+    if dtype == "fp16":
+        return np.full(want.shape, atol, np.float32)
+    mag = np.maximum(np.abs(want), np.float32(2.0 ** -126))
+    ulp = np.exp2(np.floor(np.log2(mag)) - 7).astype(np.float32)
+    return (atol + 0.5 * ulp).astype(np.float32)

@@ -1,0 +1,104 @@
+"""Workspaces and streams: the plain entry point takes its split workspace from a per-stream cache
+(nothing is allocated or filled after the first call), two streams never share one, and calls whose
+workspaces differ may overlap in time without changing a bit of their results."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import bitdecode_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+SCALE = 1.0 / math.sqrt(128)
+
+
+def _problem(device, seed, b=1, h=8, h_k=2, S=4096, R=128, bits=4, gs=128):
+    from bitladder_amd import kvcache_pack_int
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=seed)
+    kd, vd = H.to_dev(k, "fp16", device), H.to_dev(v, "fp16", device)
+    cache = H.alloc_cache(b, S, h_k, bits, gs, device)
+    kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S, "k-channel", gs, bits)
+    return H.to_dev(q, "fp16", device), cache, kd[:, S:].contiguous(), vd[:, S:].contiguous(), (q, k, v)
+
+
+def test_dropin_call_reuses_a_per_stream_workspace(device):
+    from bitladder_amd import fwd_kvcache_int, interface, plan_fwd_kvcache_int
+    q, cache, kr, vr, host = _problem(device, 11)
+    ns = 16
+    kw = dict(k_residual=kr, v_residual=vr, num_splits=ns)
+    plan = plan_fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", 128, 4, **kw)
+    want = plan.run().clone()
+    torch.cuda.synchronize()
+
+    interface._WORKSPACES.clear()
+    out1 = fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", 128, 4, **kw)
+    assert len(interface._WORKSPACES) == 1
+    (key0, ws0), = interface._WORKSPACES.items()
+    torch.cuda.synchronize()
+    allocated = torch.cuda.memory_allocated(device)
+    out_buf = torch.empty_like(q)
+    for _ in range(5):
+        out2 = fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", 128, 4, out=out_buf, **kw)
+        assert torch.equal(out2, want)
+    torch.cuda.synchronize()
+    # same buffer, nothing new allocated (the output buffer was passed in)
+    assert len(interface._WORKSPACES) == 1 and interface._WORKSPACES[key0] is ws0
+    assert torch.cuda.memory_allocated(device) == allocated + out_buf.numel() * 2
+    assert torch.equal(out1, want)
+    # the arrival counters are back at zero after every call: one 256-byte block per query head
+    counters = ws0[:256 * q.shape[0] * q.shape[2]].view(torch.int32)
+    assert int(counters.abs().sum()) == 0
+
+    # another stream gets another workspace; another split count as well
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        out3 = fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", 128, 4, **kw)
+    side.synchronize()
+    assert len(interface._WORKSPACES) == 2
+    ptrs = {ws.data_ptr() for ws in interface._WORKSPACES.values()}
+    assert len(ptrs) == 2
+    assert torch.equal(out3, want)
+    fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", 128, 4, k_residual=kr, v_residual=vr, num_splits=8)
+    assert len(interface._WORKSPACES) == 3
+
+    # and the result is the oracle's
+    qn, kn, vn = host
+    qkv = O.quantize_kv_ref(kn[:, :4096], vn[:, :4096], 4, 128)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    ref, _ = O.attend_ref(qn, k_hat, v_hat, SCALE, kn[:, 4096:], vn[:, 4096:])
+    assert np.abs(want.float().cpu().numpy() - ref).max() < 2e-3
+
+
+def test_two_plans_on_two_streams_overlap_without_changing_a_bit(device):
+    """Two plans (different problems, a workspace each) replayed many times on two streams at once give,
+    every time, the bits they give when run alone."""
+    from bitladder_amd import plan_fwd_kvcache_int
+    probs = [_problem(device, 21, h=8, h_k=2, S=8192), _problem(device, 22, h=8, h_k=1, S=4096, bits=2, gs=64)]
+    plans, wants = [], []
+    for (q, cache, kr, vr, _), (bits, gs, ns) in zip(probs, [(4, 128, 24), (2, 64, 32)]):
+        plan = plan_fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", gs, bits, k_residual=kr, v_residual=vr,
+                                    num_splits=ns, out=torch.empty_like(q))
+        plans.append(plan)
+        wants.append(plan.run().clone())
+    torch.cuda.synchronize()
+    assert plans[0].args.workspace != plans[1].args.workspace
+    streams = [torch.cuda.Stream(device), torch.cuda.Stream(device)]
+    outs = [[], []]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream(device))
+    for rep in range(40):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                plans[i].run()
+                if rep % 8 == 7:
+                    outs[i].append(plans[i].out.clone())
+    for s in streams:
+        s.synchronize()
+    for i in (0, 1):
+        assert len(outs[i]) == 5
+        for o in outs[i]:
+            assert torch.equal(o, wants[i])

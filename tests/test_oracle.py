@@ -125,6 +125,74 @@ def test_k_groups_run_along_tokens_and_v_groups_along_channels():
     assert q.k_codes[0, 5, 0, 7] == 15 and q.v_codes[0, 9, 0, 40] == 15
 
 
+# ------------------------------------------------------------------ dequantize_ref, pinned directly
+@pytest.mark.parametrize("bits,gs", [(4, 128), (4, 32), (2, 64)])
+def test_dequantize_is_exact_on_an_exact_grid_and_inverts_the_quantizer(bits, gs):
+    """Values that lie on a grid both scale and zero represent exactly come back unchanged, for K (groups
+    along tokens) and V (groups along channels) separately; a transposed or mis-repeated parameter axis
+    would put another group's scale or zero under a value and break the equality."""
+    rng = np.random.default_rng(bits * 10 + gs)
+    b, S, h, d, M = 2, 256, 2, 128, (1 << bits) - 1
+    kc = rng.integers(0, M + 1, (b, S, h, d)).astype(np.uint8)
+    vc = rng.integers(0, M + 1, (b, S, h, d)).astype(np.uint8)
+    # every group holds both end codes, so the quantizer finds the grid again
+    kc.reshape(b, S // gs, gs, h, d)[:, :, 0], kc.reshape(b, S // gs, gs, h, d)[:, :, 1] = 0, M
+    vc.reshape(b, S, h, d // gs, gs)[..., 0], vc.reshape(b, S, h, d // gs, gs)[..., 1] = 0, M
+    # a different power-of-two scale and a different zero for every group
+    k_scale = np.exp2(rng.integers(-6, 3, (b, S // gs, h, d))).astype(F32)
+    k_zero = (rng.integers(-8, 8, (b, S // gs, h, d)) * k_scale).astype(F32)
+    v_scale = np.exp2(rng.integers(-6, 3, (b, S, h, d // gs))).astype(F32)
+    v_zero = (rng.integers(-8, 8, (b, S, h, d // gs)) * v_scale).astype(F32)
+    k = kc.astype(F32) * np.repeat(k_scale, gs, axis=1) + np.repeat(k_zero, gs, axis=1)
+    v = vc.astype(F32) * np.repeat(v_scale, gs, axis=3) + np.repeat(v_zero, gs, axis=3)
+    q = O.quantize_kv_ref(k, v, bits, gs)
+    np.testing.assert_array_equal(q.k_codes, kc)
+    np.testing.assert_array_equal(q.v_codes, vc)
+    np.testing.assert_array_equal(q.k_scale, k_scale)
+    np.testing.assert_array_equal(q.v_zero, v_zero)
+    k_hat, v_hat = O.dequantize_ref(q)
+    np.testing.assert_array_equal(k_hat, k)
+    np.testing.assert_array_equal(v_hat, v)
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_dequantize_stays_within_half_a_step_of_the_input(bits):
+    """dequantize_ref(quantize_kv_ref(x)) is within scale/2 of x, plus what rounding scale to fp16 can
+    add over the code range, element by element with each element's own group scale."""
+    gs = 64
+    _, k, v = O.make_inputs(2, 2, 2, 256, 0, seed=40 + bits)
+    q = O.quantize_kv_ref(k, v, bits, gs)
+    k_hat, v_hat = O.dequantize_ref(q)
+    M = (1 << bits) - 1
+    ks = np.repeat(q.k_scale, gs, axis=1)
+    vs = np.repeat(q.v_scale, gs, axis=3)
+    assert (np.abs(k_hat - k) <= ks / 2 + M * ks * 2.0 ** -11 + 1e-6).all()
+    assert (np.abs(v_hat - v) <= vs / 2 + M * vs * 2.0 ** -11 + 1e-6).all()
+    # a group's minimum is reproduced exactly (code 0 -> zero)
+    kmin = k.reshape(2, 256 // gs, gs, 2, 128).min(axis=2)
+    np.testing.assert_array_equal(k_hat.reshape(2, 256 // gs, gs, 2, 128).min(axis=2), kmin)
+    vmin = v.reshape(2, 256, 2, 128 // gs, gs).min(axis=4)
+    np.testing.assert_array_equal(v_hat.reshape(2, 256, 2, 128 // gs, gs).min(axis=4), vmin)
+
+
+def test_dequantize_axes_with_one_hot_parameters():
+    """One non-zero scale: exactly the values of that group change, along tokens for K and along channels
+    for V."""
+    b, S, h, d, gs = 1, 128, 1, 128, 32
+    z = lambda *s: np.zeros(s, F32)
+    q = O.QuantKV(4, gs, "fp16", np.ones((b, S, h, d), np.uint8), z(b, S // gs, h, d), z(b, S // gs, h, d),
+                  np.ones((b, S, h, d), np.uint8), z(b, S, h, d // gs), z(b, S, h, d // gs))
+    q.k_scale[0, 2, 0, 17] = 3.0        # token group 2 (tokens 64..95) of channel 17
+    q.v_scale[0, 70, 0, 1] = 5.0        # channel group 1 (channels 32..63) of token 70
+    k_hat, v_hat = O.dequantize_ref(q)
+    want_k = z(b, S, h, d)
+    want_k[0, 64:96, 0, 17] = 3.0
+    want_v = z(b, S, h, d)
+    want_v[0, 70, 0, 32:64] = 5.0
+    np.testing.assert_array_equal(k_hat, want_k)
+    np.testing.assert_array_equal(v_hat, want_v)
+
+
 # ------------------------------------------------------------------ second witness (C restatement)
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("bits,gs", [(4, 128), (4, 32), (2, 64), (2, 128)])
