@@ -68,7 +68,7 @@ class FwdAppendArgs(ctypes.Structure):
 
 EXPORTS = ("bitdecode_abi_version", "bitdecode_last_error", "bitdecode_num_splits",
            "bitdecode_fwd_workspace_bytes", "bitdecode_qpack", "bitdecode_fwd",
-           "bitdecode_fwd_append", "bitdecode_fwd_append_workspace_bytes", "bitdecode_read_probe")
+           "bitdecode_fwd_append", "bitdecode_fwd_append_workspace_bytes", "bitdecode_read_probe", "bitdecode_fwd_static")
 
 _lib = None
 
@@ -101,6 +101,8 @@ def lib():
         L.bitdecode_qpack.argtypes = [ctypes.POINTER(QpackArgs), _vp]
         L.bitdecode_fwd.restype = ctypes.c_int
         L.bitdecode_fwd.argtypes = [ctypes.POINTER(FwdArgs), _vp]
+        L.bitdecode_fwd_static.restype = ctypes.c_int
+        L.bitdecode_fwd_static.argtypes = [ctypes.POINTER(FwdArgs), _vp]
         L.bitdecode_fwd_append.restype = ctypes.c_int
         L.bitdecode_fwd_append.argtypes = [ctypes.POINTER(FwdAppendArgs), _vp]
         L.bitdecode_fwd_append_workspace_bytes.restype = ctypes.c_size_t

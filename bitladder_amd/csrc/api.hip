@@ -27,6 +27,19 @@ int fail(int code, const char* fmt, ...) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Scratch of bitdecode_fwd_static: device memory that belongs to the library's code object, so the call
+// needs no allocation.  Every GPU that loads the library holds its own copy until the process ends.
+// Layout: arrival counters for up to kStaticHeads (batch x query head) rows, one 256-byte block each,
+// then the partial outputs and (max, sum) pairs of the splits.  The counter area is apart from the rest
+// for every problem size, so the zeros it is loaded with, and that every call leaves behind, hold from
+// call to call whatever the shapes.
+constexpr size_t kStaticHeads = 4096;
+constexpr size_t kStaticCounterBytes = kStaticHeads * bitdecode::kTicketStride * sizeof(int);     // 1 MiB
+constexpr size_t kStaticScratchBytes = size_t(8) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// address of `scratch` on each device (the name itself is only a host-side handle)
+unsigned char* g_scratch_ptr[64] = {};
+
 int check_quant(int bits, int gs, int dtype, int d) {
     if (d != bitdecode::kHeadDim) return fail(BITDECODE_EUNSUPPORTED, "head_dim %d unsupported (only 128)", d);
     if (bits != 2 && bits != 4) return fail(BITDECODE_EUNSUPPORTED, "num_bits %d unsupported (2 or 4)", bits);
@@ -167,7 +180,8 @@ size_t bitdecode_fwd_append_workspace_bytes(int32_t b, int32_t h, int32_t num_sp
 }
 
 // decode, or (step != null) decode step with append
-static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args* step, void* stream) {
+static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args* step, void* stream,
+                   unsigned char* static_scratch = nullptr) {
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
     if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
@@ -225,7 +239,14 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
     if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim * sizeof(float) >= (size_t(1) << 31))
         return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d heads: partial outputs of 2 GiB or more", nsplit, a->b, a->h);
-    if (nsplit > 1 || step) {
+    if (static_scratch) {
+        const size_t rows = static_cast<size_t>(a->b) * a->h;
+        const size_t need = nsplit > 1 ? static_cast<size_t>(nsplit) * rows * (kHeadDim + 2) * sizeof(float) : 0;
+        if (rows > kStaticHeads || need > kStaticScratchBytes - kStaticCounterBytes)
+            return fail(BITDECODE_EWORKSPACE, "bitdecode_fwd_static: %d splits x %zu (batch x head) rows need %zu bytes; the "
+                        "built-in scratch holds %zu rows and %zu bytes (use bitdecode_fwd with a workspace)", nsplit, rows,
+                        need, kStaticHeads, kStaticScratchBytes - kStaticCounterBytes);
+    } else if (nsplit > 1 || step) {
         const size_t need = step ? bitdecode_fwd_append_workspace_bytes(a->b, a->h, nsplit)
                                  : bitdecode_fwd_workspace_bytes(a->b, a->h, nsplit);
         if (!a->workspace || a->workspace_bytes < need)
@@ -274,7 +295,11 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
         const int64_t cap = a->block_table ? static_cast<int64_t>(a->max_pages_per_seq) * a->cache_tokens : a->cache_tokens;
         P.capacity = static_cast<int>(std::min<int64_t>(cap, INT32_MAX / 2));
     }
-    if (nsplit > 1) {
+    if (nsplit > 1 && static_scratch) {
+        P.tickets = reinterpret_cast<int*>(static_scratch);
+        P.o_part = reinterpret_cast<float*>(static_scratch + kStaticCounterBytes);
+        P.ml_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
+    } else if (nsplit > 1) {
         P.tickets = reinterpret_cast<int*>(ws);
         P.o_part = reinterpret_cast<float*>(ws + ticket_bytes(a->b, a->h));
         P.ml_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
@@ -285,6 +310,20 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
 }
 
 int bitdecode_fwd(const bitdecode_fwd_args* a, void* stream) { return run_fwd(a, nullptr, stream); }
+
+int bitdecode_fwd_static(const bitdecode_fwd_args* a, void* stream) {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess || dev < 0 || dev >= 64)
+        return fail(BITDECODE_ELAUNCH, "bitdecode_fwd_static: no current device (%s)", hipGetErrorString(e));
+    unsigned char* ptr = g_scratch_ptr[dev];
+    if (!ptr) {
+        // once per device, with that device current: where this device keeps its copy of the array
+        if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)); e != hipSuccess || !ptr)
+            return fail(BITDECODE_ELAUNCH, "bitdecode_fwd_static: address of the built-in scratch: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    return run_fwd(a, nullptr, stream, ptr);
+}
 
 int bitdecode_fwd_append(const bitdecode_fwd_append_args* a, void* stream) {
     if (!a) return fail(BITDECODE_EINVAL, "args is null");

@@ -111,6 +111,16 @@ typedef struct bitdecode_fwd_args {
 
 int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
 
+/* bitdecode_fwd for callers that cannot allocate device memory (code under HIP-graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * results as bitdecode_fwd, except that `workspace` / `workspace_bytes` are ignored: partial outputs and
+ * arrival counters live in an 8 MiB array inside the library's code object (one copy per GPU, held until the
+ * process ends), and the call allocates nothing.  Limits: b * h <= 4096 and num_splits * b * h * 520 bytes
+ * <= 7 MiB, otherwise BITDECODE_EWORKSPACE.  All calls on one GPU share that array: calls that overlap in
+ * time on one GPU (two streams, two host threads) race; calls on one stream do not.  The first call on a
+ * device looks up the array's address (hipGetSymbolAddress): make it outside any stream capture. */
+int bitdecode_fwd_static(const bitdecode_fwd_args* args, void* stream);
+
 /* One decode step in one launch: attend the new token together with everything held, append it, and
  * quantize-pack the fp16 window when it fills.  This is the "residual kernel" the reference's figures
  * describe (imgs/overview.png, imgs/scheme.png) and its kernel traits still name
