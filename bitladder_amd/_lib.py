@@ -10,8 +10,9 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbitdecode.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 FP16, BF16 = 0, 1
+K_CHANNEL, K_TENSOR = 0, 1
 
 _i32, _i64, _vp, _f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
 
@@ -28,6 +29,7 @@ class QpackArgs(ctypes.Structure):
         ("bits", _i32), ("group_size", _i32), ("dtype", _i32),
         ("block_table", _vp), ("block_table_stride", _i64),
         ("max_pages_per_seq", _i32), ("num_pages", _i32),
+        ("quant_mode", _i32),
     ]
 
 
@@ -52,6 +54,7 @@ class FwdArgs(ctypes.Structure):
         ("num_splits", _i32),
         ("block_table", _vp), ("block_table_stride", _i64),
         ("max_pages_per_seq", _i32), ("num_pages", _i32),
+        ("quant_mode", _i32),
     ]
 
 

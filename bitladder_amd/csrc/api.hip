@@ -50,6 +50,16 @@ int check_quant(int bits, int gs, int dtype, int d) {
     return 0;
 }
 
+int check_mode(int quant_mode, int bits, bool step) {
+    if (quant_mode != BITDECODE_K_CHANNEL && quant_mode != BITDECODE_K_TENSOR)
+        return fail(BITDECODE_EINVAL, "quant_mode %d (k-channel=0, k-tensor=1)", quant_mode);
+    if (quant_mode == BITDECODE_K_TENSOR && bits != 4)
+        return fail(BITDECODE_EUNSUPPORTED, "quant_mode k-tensor is implemented for 4 bits only (as in the reference)");
+    if (quant_mode == BITDECODE_K_TENSOR && step)
+        return fail(BITDECODE_EUNSUPPORTED, "the decode step with append is not implemented for quant_mode k-tensor");
+    return 0;
+}
+
 int query_cus() {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -118,6 +128,7 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
     if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
+    if (int rc = check_mode(a->quant_mode, a->bits, false)) return rc;
     if (a->b < 0 || a->h_k <= 0 || a->n_tokens < 0) return fail(BITDECODE_EINVAL, "negative size");
     if (a->n_tokens % kChunk) return fail(BITDECODE_EINVAL, "n_tokens %d is not a multiple of 128", a->n_tokens);
     if (a->cache_tokens % kChunk || a->cache_tokens <= 0)
@@ -159,7 +170,9 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     P.v_params = static_cast<uint8_t*>(a->v_params);
     P.kpack_bh = code_region_bytes(a->cache_tokens, a->bits);
     P.vpack_bh = P.kpack_bh;
-    P.kparams_bh = k_param_region_bytes(a->cache_tokens, a->group_size);
+    P.ktensor = a->quant_mode == BITDECODE_K_TENSOR;
+    P.kparams_bh = P.ktensor ? v_param_region_bytes(a->cache_tokens, a->group_size)
+                             : k_param_region_bytes(a->cache_tokens, a->group_size);
     P.vparams_bh = v_param_region_bytes(a->cache_tokens, a->group_size);
     P.b = a->b; P.n_tokens = a->n_tokens; P.hk = a->h_k;
     P.dst_offset = a->dst_offset;
@@ -185,6 +198,7 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
     if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
+    if (int rc = check_mode(a->quant_mode, a->bits, step != nullptr)) return rc;
     if (a->b <= 0 || a->h <= 0 || a->h_k <= 0) return fail(BITDECODE_EINVAL, "batch and head counts must be positive");
     if (a->h % a->h_k) return fail(BITDECODE_EINVAL, "h %d is not a multiple of h_k %d", a->h, a->h_k);
     const int g = a->h / a->h_k;
@@ -264,7 +278,9 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     P.v_params = static_cast<const uint8_t*>(a->v_params);
     P.kpack_bh = code_region_bytes(a->cache_tokens, a->bits);
     P.vpack_bh = P.kpack_bh;
-    P.kparams_bh = k_param_region_bytes(a->cache_tokens, a->group_size);
+    P.ktensor = a->quant_mode == BITDECODE_K_TENSOR;
+    P.kparams_bh = P.ktensor ? v_param_region_bytes(a->cache_tokens, a->group_size)
+                             : k_param_region_bytes(a->cache_tokens, a->group_size);
     P.vparams_bh = v_param_region_bytes(a->cache_tokens, a->group_size);
     P.k_res = static_cast<const uint16_t*>(a->k_res);
     P.v_res = static_cast<const uint16_t*>(a->v_res);

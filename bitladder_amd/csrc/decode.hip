@@ -329,6 +329,7 @@ struct UnitCfg {
     static constexpr int NCG = kHeadDim / GS;                // V channel groups
     static constexpr int KPB = unit_k_param_bytes(BITS, GS); // K parameter bytes per unit
     static constexpr int VPB = unit_v_param_bytes(BITS, GS); // V parameter bytes per unit
+    static constexpr int KPB_T = UT * NCG * 4;                // K parameter bytes per unit in "k-tensor" mode (per token)
     static constexpr int NKP = (KPB + 1023) / 1024;          // load instructions for the K parameters
     static constexpr int NVP = (VPB + 1023) / 1024;          // ... for the V parameters
     static constexpr int KSIDE = NKP + 4;                    // loads of a unit's K side (parameters, 4 code rows)
@@ -339,6 +340,7 @@ struct UnitCfg {
     static constexpr int NW = decode_waves(BITS, GS);        // waves per workgroup
     static constexpr int DEPTH = (X_DEPTH) < NKP + RPS + 1 ? (X_DEPTH) : NKP + RPS + 1;   // rows a wave keeps in flight
     static_assert(REGION == OFF_VP + VPB && REGION % 256 == 0, "region layout");
+    static_assert(KPB_T <= KPB && (KPB_T + 1023) / 1024 == NKP, "the per-token K parameters use the same rows");
     static_assert(NW % 4 == 0, "the merge reads four wave weights per LDS access");
 };
 
@@ -454,7 +456,7 @@ struct UnitAddr {
     const uint8_t* kp;
     const uint8_t* vp;
 };
-template <int BITS, int GS>
+template <int BITS, int GS, bool KT = false>
 __device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int bi, int hk, int u) {
     using C = UnitCfg<BITS, GS>;
     const int uic = u % C::UPC;
@@ -474,8 +476,12 @@ __device__ __forceinline__ UnitAddr<BITS, GS> unit_addr(const FwdParams& P, int 
     UnitAddr<BITS, GS> A;      // wave-uniform: everything here lives in SGPRs
     A.kc = P.k_pack + bh * P.kpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
     A.vc = P.v_pack + bh * P.vpack_bh + static_cast<int64_t>(ci) * chunk_code_bytes(BITS) + uic * 4096;
-    A.kp = P.k_params + bh * P.kparams_bh +
-           (static_cast<int64_t>(ci) * (kChunk / GS) + (uic * C::UT) / GS) * kKParamGroupBytes;
+    if constexpr (KT) {      // per-token K parameters: [64-token half][channel group][tile][token] per chunk
+        A.kp = P.k_params + bh * P.kparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS) + uic * C::KPB_T;
+    } else {
+        A.kp = P.k_params + bh * P.kparams_bh +
+               (static_cast<int64_t>(ci) * (kChunk / GS) + (uic * C::UT) / GS) * kKParamGroupBytes;
+    }
     A.vp = P.v_params + bh * P.vparams_bh + static_cast<int64_t>(ci) * v_param_chunk_bytes(GS) + uic * C::VPB;
     return A;
 }
@@ -539,13 +545,13 @@ constexpr int pos_of(int kind, int idx) {
     return -1;
 }
 // the load of row I of a unit into the wave's region; kslot names the K-parameter slot of that unit
-template <int BITS, int GS, int I>
+template <int BITS, int GS, int I, bool KT = false>
 __device__ __forceinline__ void issue_row(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region, int kslot) {
     using C = UnitCfg<BITS, GS>;
     constexpr RowId r = row_at<BITS, GS>(I);
     static_assert(r.kind >= 0, "row inside the unit");
     if constexpr (r.kind == 0) {
-        constexpr int left = C::KPB - r.idx * 1024;
+        constexpr int left = (KT ? C::KPB_T : C::KPB) - r.idx * 1024;
         const uint32_t dst = region + C::OFF_KP + kslot * C::KPB;
         if constexpr (left >= 1024) {
             dma_row<r.idx * 1024>(A.kp, lane16, dst);
@@ -566,18 +572,18 @@ __device__ __forceinline__ void issue_row(const UnitAddr<BITS, GS>& A, uint32_t 
     }
 }
 // prologue of a wave: rows 0 .. kDepth-2 of its first unit
-template <int BITS, int GS, int I = 0>
+template <int BITS, int GS, bool KT = false, int I = 0>
 __device__ __forceinline__ void issue_first_rows(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region) {
     if constexpr (I < UnitCfg<BITS, GS>::DEPTH - 1) {
-        issue_row<BITS, GS, I>(A, lane16, region, 0);
-        issue_first_rows<BITS, GS, I + 1>(A, lane16, region);
+        issue_row<BITS, GS, I, KT>(A, lane16, region, 0);
+        issue_first_rows<BITS, GS, KT, I + 1>(A, lane16, region);
     }
 }
 // In front of the read of row I of the current unit: send the row that keeps the pipeline full (of this
 // unit, or of the next one if there is one), then wait until row I has landed.  The load may overwrite
 // rows read earlier: every LDS read issued so far has to have returned its data first (a read that has
 // only been issued can be overtaken by the load's write).
-template <int BITS, int GS, bool HAS_NEXT, int I>
+template <int BITS, int GS, bool HAS_NEXT, int I, bool KT = false>
 __device__ __forceinline__ void row_ready(const UnitAddr<BITS, GS>& cur, const UnitAddr<BITS, GS>& next, uint32_t lane16,
                                           uint32_t region, int kslot) {
     using C = UnitCfg<BITS, GS>;
@@ -587,11 +593,11 @@ __device__ __forceinline__ void row_ready(const UnitAddr<BITS, GS>& cur, const U
     static_assert(kDepth - 1 <= C::NKP + C::RPS && kDepth - 1 < ROWS, "depth of the row pipeline");
     if constexpr (J < ROWS) {
         wait_lds_reads();
-        issue_row<BITS, GS, J>(cur, lane16, region, kslot);
+        issue_row<BITS, GS, J, KT>(cur, lane16, region, kslot);
         wait_vm<kDepth - 1>();
     } else if constexpr (HAS_NEXT) {
         wait_lds_reads();
-        issue_row<BITS, GS, J - ROWS>(next, lane16, region, kslot ^ 1);
+        issue_row<BITS, GS, J - ROWS, KT>(next, lane16, region, kslot ^ 1);
         wait_vm<kDepth - 1>();
     } else {
         wait_vm<ROWS - 1 - I>();
@@ -652,11 +658,44 @@ __device__ __forceinline__ void start_group(KGroup& G, const uint8_t* kpar, cons
 // scale is applied inside the exponent.  On entry rows 0 .. kDepth-2 of the unit are in flight or landed;
 // with HAS_NEXT the first rows of the wave's next unit are issued from here (see above); kslot says
 // which K-parameter slot the current unit uses.
-template <int BITS, int GS, bool BF16, bool HAS_NEXT>
+// With KT ("k-tensor" mode: K parameters per token and channel group) the K scale cannot be folded into q:
+// a tile's raw sums  sum_c (offset + code) q_c  are taken per channel group with q as it is (hi columns
+// only: q is exact in fp16), and each of the tile's tokens then applies its own scale and zero,
+//   score = sum_g scale_g * (raw_g - sum_c offset_c q_c) + zero_g * sum_c q_c   (c in group g),
+// with the two q sums of every group prepared once per wave (KQ).
+template <int NCG>
+struct TokenQ {
+    h8 q[4];          // q of the lane's head in the hi columns, zero in the lo columns
+    float noffq[NCG]; // - sum_c offset_c q_c per channel group, for the lane's column
+    float qsum[NCG];  //   sum_c q_c
+};
+template <int BITS, int NCG>
+__device__ __forceinline__ TokenQ<NCG> token_q(const QRows& Q) {
+    TokenQ<NCG> T;
+    const h8 noff = -code_offsets<BITS>();
+    const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
+    f4 no[NCG], qs[NCG];       // every row of these products is the same
+#pragma unroll
+    for (int c = 0; c < NCG; ++c) no[c] = qs[c] = f4{0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        T.q[j] = q_load(Q.qz, j);
+        no[j * NCG / 4] = mfma32(noff, T.q[j], no[j * NCG / 4]);
+        qs[j * NCG / 4] = mfma32(ones, T.q[j], qs[j * NCG / 4]);
+    }
+#pragma unroll
+    for (int c = 0; c < NCG; ++c) {
+        T.noffq[c] = no[c][0];
+        T.qsum[c] = qs[c][0];
+    }
+    return T;
+}
+
+template <int BITS, int GS, bool BF16, bool HAS_NEXT, bool KT = false>
 __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, int kslot,
                                              const UnitAddr<BITS, GS>& cur, const UnitAddr<BITS, GS>& next,
                                              const QRows& Q, const FwdParams& P, int lane, bool lo_part, const Magic& mg,
-                                             WaveState<kHeadDim / GS>& st) {
+                                             WaveState<kHeadDim / GS>& st, const TokenQ<kHeadDim / GS>* KQ = nullptr) {
     using C = UnitCfg<BITS, GS>;
     constexpr int NCG = C::NCG, TPS = C::TPS, NKS = C::NKS, TPG = C::TPG, CTPG = GS / 16;
     constexpr int NSTEP = C::NSTEP, RPS = C::RPS, TPR = TPS / RPS;      // tiles per K row
@@ -669,7 +708,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     const u4* vcode = reinterpret_cast<const u4*>(reg + 4096) + lane;
     const uint8_t* kpar = reg + C::OFF_KP + kslot * C::KPB;
     const uint8_t* vpar = reg + C::OFF_VP + kg * 16;
-#define ROW_READY(kind, idx) row_ready<BITS, GS, HAS_NEXT, pos_of<BITS, GS>(kind, idx)>(cur, next, lane16, region_lds, kslot)
+#define ROW_READY(kind, idx) row_ready<BITS, GS, HAS_NEXT, pos_of<BITS, GS>(kind, idx), KT>(cur, next, lane16, region_lds, kslot)
 
     // the K parameters lead the queue: the first K group is prepared while the code rows arrive
 #pragma unroll
@@ -679,7 +718,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     }
     static_assert(C::NKP <= 2 && C::NVP <= 2, "parameter rows of a unit");
     KGroup G;
-    start_group<BITS, BF16>(G, kpar, Q, kg);
+    if constexpr (!KT) start_group<BITS, BF16>(G, kpar, Q, kg);
 #pragma unroll
     for (int step = 0; step < NSTEP; ++step) {
         f4 sc[TPS];
@@ -692,6 +731,28 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
                 if (row == 1) ROW_READY(1, 1);
                 if (row == 2) ROW_READY(1, 2);
                 if (row == 3) ROW_READY(1, 3);
+            }
+            if constexpr (KT) {
+                static_assert(!KT || BITS == 4, "per-token K parameters: 4 bits only");
+                const u4 w = kcode[64 * tile];
+                f4 raw[NCG];
+#pragma unroll
+                for (int c = 0; c < NCG; ++c) raw[c] = f4{KQ->noffq[c], KQ->noffq[c], KQ->noffq[c], KQ->noffq[c]};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw[j * NCG / 4] = mfma32(dq4(w[j], mg), KQ->q[j], raw[j * NCG / 4]);
+                f4 acc = {0, 0, 0, 0};
+#pragma unroll
+                for (int c = 0; c < NCG; ++c) {
+                    // (scale, zero) of the tile's tokens 4*kg .. 4*kg+3 for channel group c
+                    const h8 pr = *reinterpret_cast<const h8*>(kpar + (c * 4 + tile) * 64 + kg * 16);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        acc[r] = __builtin_fmaf(static_cast<float>(pr[2 * r]), raw[c][r],
+                                                __builtin_fmaf(static_cast<float>(pr[2 * r + 1]), KQ->qsum[c], acc[r]));
+                    }
+                }
+                sc[tt] = acc;
+                continue;
             }
             if (tile != 0 && tile % TPG == 0) {
                 start_group<BITS, BF16>(G, kpar + ((tile * 16) / GS) * kKParamGroupBytes, Q, kg);
@@ -1165,8 +1226,9 @@ constexpr int fwd_lds_bytes() {
     return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16;
 }
 
-template <int BITS, int GS, bool BF16, bool APPEND>
+template <int BITS, int GS, bool BF16, bool APPEND, bool KT>
 __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
+    static_assert(!KT || (BITS == 4 && !APPEND), "per-token K parameters: 4 bits, plain decode");
     using C = UnitCfg<BITS, GS>;
     constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -1237,8 +1299,8 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     }
     UnitAddr<BITS, GS> A;
     if (u < u1) {
-        A = unit_addr<BITS, GS>(P, bi, hk, u);
-        issue_first_rows<BITS, GS>(A, lane * 16, region_lds);
+        A = unit_addr<BITS, GS, KT>(P, bi, hk, u);
+        issue_first_rows<BITS, GS, KT>(A, lane * 16, region_lds);
         wait_then_take<C::DEPTH - 1>(qa, qb, qa_raw, qb_raw);
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
@@ -1275,14 +1337,20 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         wait_vm<C::DEPTH - 2>();   // first row (K parameters) has arrived
         PROF(2);
 #endif
+        TokenQ<NCG> KQ;
+        const TokenQ<NCG>* KQp = nullptr;
+        if constexpr (KT) {
+            KQ = token_q<BITS, NCG>(Q);
+            KQp = &KQ;
+        }
         int kslot = 0;
         for (int un = u + NW; un < u1; un += NW) {        // units that have a successor: it is fetched from inside
-            const UnitAddr<BITS, GS> An = unit_addr<BITS, GS>(P, bi, hk, un);
-            compute_unit<BITS, GS, BF16, true>(region, region_lds, kslot, A, An, Q, P, lane, lo_part, mg, st);
+            const UnitAddr<BITS, GS> An = unit_addr<BITS, GS, KT>(P, bi, hk, un);
+            compute_unit<BITS, GS, BF16, true, KT>(region, region_lds, kslot, A, An, Q, P, lane, lo_part, mg, st, KQp);
             A = An;
             kslot ^= 1;
         }
-        compute_unit<BITS, GS, BF16, false>(region, region_lds, kslot, A, A, Q, P, lane, lo_part, mg, st);
+        compute_unit<BITS, GS, BF16, false, KT>(region, region_lds, kslot, A, A, Q, P, lane, lo_part, mg, st, KQp);
     }
     PROF(3);
     // ---- fp16 window tiles of this wave (the region becomes the V-transpose slab)
@@ -1434,7 +1502,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     PROF_FLUSH();
 }
 
-template <int BITS, int GS, bool BF16, bool APPEND>
+template <int BITS, int GS, bool BF16, bool APPEND, bool KT = false>
 hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
     constexpr int kLds = fwd_lds_bytes<BITS, GS>();
     // the dynamic-LDS limit is raised once per kernel and device (idempotent, so a race between
@@ -1443,18 +1511,27 @@ hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !configured[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16, APPEND>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return e;
         if (dev >= 0 && dev < 64) configured[dev] = true;
     }
-    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16, APPEND>), dim3(P.nsplit * P.hk * P.b),
+    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT>), dim3(P.nsplit * P.hk * P.b),
                        dim3(UnitCfg<BITS, GS>::NW * 64), kLds, stream, P);
     return hipGetLastError();
 }
 
 template <int BITS, int GS>
 hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
+    if (P.ktensor) {      // "k-tensor" mode: 4 bits, plain decode
+        if constexpr (BITS == 4) {
+            if (P.lengths) return hipErrorInvalidValue;
+            return P.bf16 ? launch_fwd_tt<BITS, GS, true, false, true>(P, stream)
+                          : launch_fwd_tt<BITS, GS, false, false, true>(P, stream);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
     if (P.lengths) {
         return P.bf16 ? launch_fwd_tt<BITS, GS, true, true>(P, stream) : launch_fwd_tt<BITS, GS, false, true>(P, stream);
     }

@@ -12,7 +12,7 @@
 namespace bitdecode {
 namespace {
 
-template <int BITS, int GS, bool BF16>
+template <int BITS, int GS, bool BF16, bool KT>
 __global__ __launch_bounds__(qp::kPackThreads) void qpack_kernel(QpackParams P) {
     __shared__ qp::PackLds<GS> L;
     const int tid = threadIdx.x;
@@ -21,7 +21,7 @@ __global__ __launch_bounds__(qp::kPackThreads) void qpack_kernel(QpackParams P) 
     if (dst_base < 0) return;       // a negative per-sequence offset skips that sequence (whole workgroup)
     const int dst_tok = dst_base + ci_src * kChunk;
     const ChunkPlace place = chunk_place(P.block_table, P.bt_stride, P.chunks_per_page, bi, hk, P.hk, dst_tok / kChunk);
-    const qp::ChunkDst D = qp::chunk_dst<BITS, GS>(P.k_pack, P.k_params, P.v_pack, P.v_params, P.kpack_bh, P.kparams_bh,
+    const qp::ChunkDst D = qp::chunk_dst<BITS, GS, KT>(P.k_pack, P.k_params, P.v_pack, P.v_params, P.kpack_bh, P.kparams_bh,
                                                    P.vpack_bh, P.vparams_bh, place);
     const uint16_t* ks = P.k + bi * P.k_sb + static_cast<int64_t>(ci_src) * kChunk * P.k_st + hk * P.k_sh;
     const uint16_t* vs = P.v + bi * P.v_sb + static_cast<int64_t>(ci_src) * kChunk * P.v_st + hk * P.v_sh;
@@ -29,17 +29,29 @@ __global__ __launch_bounds__(qp::kPackThreads) void qpack_kernel(QpackParams P) 
     // 4 bits, group 128: with the V tile prefetched the kernel needs 133 registers and only three
     // workgroups fit a CU; fetched after the K side it needs 114, a fourth workgroup fits (LDS: 40 KB
     // each) and the kernel is 10 % faster.  (At group 64 a fourth workgroup was measured 3 % slower.)
-    qp::pack_chunk<BITS, GS, BF16, !(BITS == 4 && GS == 128)>(
+    qp::pack_chunk<BITS, GS, BF16, !(BITS == 4 && GS == 128), KT>(
         L, tid, true, [=](int n) { return ks + n * k_st; }, [=](int n) { return vs + n * v_st; }, D);
 }
 
 template <int BITS, int GS>
 hipError_t launch_qpack_t(const QpackParams& P, hipStream_t stream) {
     dim3 grid(P.n_tokens / kChunk, P.hk, P.b);
+    if (P.ktensor) {      // K quantized per token like V: 4 bits only, as in the reference (qpack.h:385)
+        if constexpr (BITS == 4) {
+            if (P.bf16) {
+                hipLaunchKernelGGL((qpack_kernel<BITS, GS, true, true>), grid, dim3(256), 0, stream, P);
+            } else {
+                hipLaunchKernelGGL((qpack_kernel<BITS, GS, false, true>), grid, dim3(256), 0, stream, P);
+            }
+            return hipGetLastError();
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
     if (P.bf16) {
-        hipLaunchKernelGGL((qpack_kernel<BITS, GS, true>), grid, dim3(256), 0, stream, P);
+        hipLaunchKernelGGL((qpack_kernel<BITS, GS, true, false>), grid, dim3(256), 0, stream, P);
     } else {
-        hipLaunchKernelGGL((qpack_kernel<BITS, GS, false>), grid, dim3(256), 0, stream, P);
+        hipLaunchKernelGGL((qpack_kernel<BITS, GS, false, false>), grid, dim3(256), 0, stream, P);
     }
     return hipGetLastError();
 }

@@ -98,14 +98,15 @@ struct ChunkDst {
     uint8_t* vc;
     uint8_t* vp;
 };
-template <int BITS, int GS>
+template <int BITS, int GS, bool KT = false>
 __device__ __forceinline__ ChunkDst chunk_dst(uint8_t* k_pack, uint8_t* k_params, uint8_t* v_pack, uint8_t* v_params,
                                               int64_t kpack_bh, int64_t kparams_bh, int64_t vpack_bh,
                                               int64_t vparams_bh, const ChunkPlace& place) {
     const int64_t bh = place.region, ci = place.chunk;
     ChunkDst D;
     D.kc = k_pack + bh * kpack_bh + ci * chunk_code_bytes(BITS);
-    D.kp = k_params + bh * kparams_bh + ci * (kChunk / GS) * kKParamGroupBytes;
+    // ("k-tensor": K parameters per token and channel group, as many bytes per chunk as V's)
+    D.kp = k_params + bh * kparams_bh + ci * (KT ? v_param_chunk_bytes(GS) : (kChunk / GS) * kKParamGroupBytes);
     D.vc = v_pack + bh * vpack_bh + ci * chunk_code_bytes(BITS);
     D.vp = v_params + bh * vparams_bh + ci * v_param_chunk_bytes(GS);
     return D;
@@ -118,7 +119,43 @@ __device__ __forceinline__ ChunkDst chunk_dst(uint8_t* k_pack, uint8_t* k_params
 // 32 registers free), per-channel statistics are taken column-wise, per-token statistics row-wise,
 // and each thread then assembles whole 16-byte lane slots of the packed layout so that the stores
 // are full 1 KB wave rows.
-template <int BITS, int GS, bool BF16, bool PREFETCH_V, class RowK, class RowV>
+// Minimum and maximum of every (token, channel group) of the tile in LDS: thread -> token tid/2, 64-channel
+// half tid%2.  store(n, cg, mn, mx) is called once per group by the thread that holds its statistics.
+template <int GS, bool BF16, class Store>
+__device__ __forceinline__ void row_group_stats(const uint16_t* tile, int tid, Store store) {
+    const int n = tid >> 1, hf = tid & 1;   // token, 64-channel half
+    constexpr int PARTS = (GS >= 64) ? 1 : 2;        // groups fully inside this thread's half
+    constexpr int PW = 64 / PARTS;                   // channels per part
+    float pmn[PARTS], pmx[PARTS];
+#pragma unroll
+    for (int pt = 0; pt < PARTS; ++pt) {
+        const uint16_t* row = &tile[n * kRowHalves + 64 * hf + PW * pt];
+        float mn = to_f32<BF16>(row[0]), mx = mn;
+#pragma unroll
+        for (int c = 1; c < PW; ++c) {
+            float x = to_f32<BF16>(row[c]);
+            mn = fminf(mn, x);
+            mx = fmaxf(mx, x);
+        }
+        pmn[pt] = mn;
+        pmx[pt] = mx;
+    }
+    if constexpr (GS == 128) {
+        pmn[0] = fminf(pmn[0], __shfl_xor(pmn[0], 1));
+        pmx[0] = fmaxf(pmx[0], __shfl_xor(pmx[0], 1));
+    }
+#pragma unroll
+    for (int pt = 0; pt < PARTS; ++pt) {
+        const int cg = (GS == 128) ? 0 : (GS == 64 ? hf : 2 * hf + pt);
+        if (GS == 128 && hf != 0) break;
+        store(n, cg, pmn[pt], pmx[pt]);
+    }
+}
+
+// With KT ("k-tensor" mode, qpack.h:378-470 of the reference) K is quantized like V, per token over groups
+// of GS channels; its codes keep the K layout, its parameters go per chunk as
+// [64-token half][channel group][16-token tile][token] (scale, zero) pairs.
+template <int BITS, int GS, bool BF16, bool PREFETCH_V, bool KT = false, class RowK, class RowV>
 __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active, RowK krow, RowV vrow,
                                            const ChunkDst& D) {
 #pragma clang fp contract(off)
@@ -141,8 +178,23 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
     }
     __syncthreads();
 
-    // ================= K: per-channel groups of GS tokens =================
-    if (active) {
+    // ================= K: per-channel groups of GS tokens (KT: per-token groups of GS channels) =================
+    if constexpr (KT) {
+        if (active) {
+            row_group_stats<GS, BF16>(tile, tid, [&](int n, int cg, float mn, float mx) {
+                float sinv, scale;
+                group_params(mn, mx, M, sinv, scale);
+                L.v_sinv[n][cg] = sinv;
+                L.v_mn[n][cg] = mn;
+                uint16_t* dst = reinterpret_cast<uint16_t*>(
+                    D.kp + ((((n >> 6) * NCG + cg) * 4 + ((n >> 4) & 3)) * 16 + (n & 15)) * 4);
+                dst[0] = param_bits<BF16>(scale);
+                dst[1] = param_bits<BF16>(mn);
+            });
+        }
+        __syncthreads();
+    }
+    if (!KT && active) {
         const int c = tid & 127, part = tid >> 7;
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq) {
@@ -159,8 +211,8 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
             L.k_qmax[quarter][c] = mx;
         }
     }
-    __syncthreads();
-    if (active) {
+    if constexpr (!KT) __syncthreads();
+    if (!KT && active) {
         for (int idx = tid; idx < NG * kHeadDim; idx += kPackThreads) {
             const int grp = idx >> 7, c = idx & 127;
             constexpr int QPG = GS / 32;  // quarters per group
@@ -179,7 +231,7 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
             kp[kHeadDim + c] = param_bits<BF16>(mn);
         }
     }
-    __syncthreads();
+    if constexpr (!KT) __syncthreads();
     if (active) {
         uint8_t* const kc = D.kc;
         if constexpr (BITS == 4) {
@@ -196,7 +248,8 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         float x = to_f32<BF16>(tile[n * kRowHalves + ch0 + i]);
-                        uint32_t code = quant_code(x, L.k_mn[grp][ch0 + i], L.k_sinv[grp][ch0 + i]);
+                        uint32_t code = KT ? quant_code(x, L.v_mn[n][(ch0 + i) / GS], L.v_sinv[n][(ch0 + i) / GS])
+                                           : quant_code(x, L.k_mn[grp][ch0 + i], L.k_sinv[grp][ch0 + i]);
                         const int p = i / 2 + 4 * (i % 2);
                         w |= code << (4 * p);
                     }
@@ -218,7 +271,8 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
                         const int j = 2 * jj + e / 8, i = e % 8;
                         const int ch = 32 * j + 8 * kg + i;
                         float x = to_f32<BF16>(tile[n * kRowHalves + ch]);
-                        uint32_t code = quant_code(x, L.k_mn[grp][ch], L.k_sinv[grp][ch]);
+                        uint32_t code = KT ? quant_code(x, L.v_mn[n][ch / GS], L.v_sinv[n][ch / GS])
+                                           : quant_code(x, L.k_mn[grp][ch], L.k_sinv[grp][ch]);
                         const int f = e / 2 + 8 * (e % 2);
                         w |= code << (2 * f);
                     }
@@ -241,40 +295,16 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
     }
     __syncthreads();
     if (active) {
-        const int n = tid >> 1, hf = tid & 1;   // token, 64-channel half
-        constexpr int PARTS = (GS >= 64) ? 1 : 2;        // groups fully inside this thread's half
-        constexpr int PW = 64 / PARTS;                   // channels per part
-        float pmn[PARTS], pmx[PARTS];
-#pragma unroll
-        for (int pt = 0; pt < PARTS; ++pt) {
-            const uint16_t* row = &tile[n * kRowHalves + 64 * hf + PW * pt];
-            float mn = to_f32<BF16>(row[0]), mx = mn;
-#pragma unroll
-            for (int c = 1; c < PW; ++c) {
-                float x = to_f32<BF16>(row[c]);
-                mn = fminf(mn, x);
-                mx = fmaxf(mx, x);
-            }
-            pmn[pt] = mn;
-            pmx[pt] = mx;
-        }
-        if constexpr (GS == 128) {
-            pmn[0] = fminf(pmn[0], __shfl_xor(pmn[0], 1));
-            pmx[0] = fmaxf(pmx[0], __shfl_xor(pmx[0], 1));
-        }
-        const int sb = n >> 5, T = (n >> 4) & 1, q = (n >> 2) & 3, r = n & 3, i = 4 * T + r;
-#pragma unroll
-        for (int pt = 0; pt < PARTS; ++pt) {
-            const int cg = (GS == 128) ? 0 : (GS == 64 ? hf : 2 * hf + pt);
-            if (GS == 128 && hf != 0) break;
+        row_group_stats<GS, BF16>(tile, tid, [&](int n, int cg, float mn, float mx) {
+            const int sb = n >> 5, T = (n >> 4) & 1, q = (n >> 2) & 3, r = n & 3, i = 4 * T + r;
             float sinv, scale;
-            group_params(pmn[pt], pmx[pt], M, sinv, scale);
+            group_params(mn, mx, M, sinv, scale);
             L.v_sinv[n][cg] = sinv;
-            L.v_mn[n][cg] = pmn[pt];
+            L.v_mn[n][cg] = mn;
             uint16_t* dst = reinterpret_cast<uint16_t*>(D.vp + (sb * NCG + cg) * 128 + q * 16 + i * 2);
             dst[0] = param_bits<BF16>(scale);
-            dst[32] = param_bits<BF16>(pmn[pt]);   // zeros start 64 bytes after the scales
-        }
+            dst[32] = param_bits<BF16>(mn);   // zeros start 64 bytes after the scales
+        });
     }
     __syncthreads();
     if (active) {

@@ -25,14 +25,18 @@ def _dtype_code(t: torch.Tensor) -> int:
     raise RuntimeError("bit_decode only supports fp16 and bf16 data type")
 
 
-def _check_quant(quant_mode: str, group_size: int, num_bits: int) -> None:
-    if quant_mode != "k-channel":
-        # the reference's "k-tensor" instantiations are commented out (decode_api.cpp:195-203)
-        raise NotImplementedError(f"quant_mode {quant_mode!r} is not supported (only 'k-channel')")
+def _check_quant(quant_mode: str, group_size: int, num_bits: int) -> int:
+    """Returns the C ABI's code of the quantization mode."""
+    if quant_mode not in ("k-channel", "k-tensor"):
+        raise ValueError(f"quant_mode must be 'k-channel' or 'k-tensor', got {quant_mode!r}")
     if num_bits not in (2, 4):
         raise ValueError(f"num_bits must be 2 or 4, got {num_bits}")
     if group_size not in (32, 64, 128):
         raise ValueError(f"group_size must be 32, 64 or 128, got {group_size}")
+    if quant_mode == "k-tensor" and num_bits != 4:
+        # the reference's quantizer for this mode is 4-bit only (qpack.h:385)
+        raise NotImplementedError("quant_mode 'k-tensor' is implemented for num_bits=4 only")
+    return _lib.K_TENSOR if quant_mode == "k-tensor" else _lib.K_CHANNEL
 
 
 def _check_block_table(block_table, b, device):
@@ -55,9 +59,10 @@ def _set_paging(a, block_table, num_pages):
     a.num_pages = num_pages
 
 
-def _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device):
+def _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device, k_tensor=False):
     """Validates the caller-allocated packed tensors (evaluation/test.py:74-83) and returns
-    (batch, capacity_tokens, h_k)."""
+    (batch, capacity_tokens, h_k).  In "k-tensor" mode K has one (scale, zero) per token and channel
+    group, and k_params has v_params' shape."""
     pn = 16 // num_bits
     if v_pack.dim() != 4 or k_pack.dim() != 4 or k_params.dim() != 4 or v_params.dim() != 4:
         raise RuntimeError("k_pack, k_params, v_pack, v_params must be 4-dimensional")
@@ -68,7 +73,8 @@ def _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, devic
     if S % CHUNK:
         raise RuntimeError(f"packed cache capacity {S} must be a multiple of {CHUNK} tokens")
     want = {
-        "k_pack": (b, S // pn, h_k, d), "k_params": (b, S // group_size, h_k, d),
+        "k_pack": (b, S // pn, h_k, d),
+        "k_params": (b, d // group_size, h_k, S) if k_tensor else (b, S // group_size, h_k, d),
         "v_pack": (b, S, h_k, d // pn), "v_params": (b, d // group_size, h_k, S),
     }
     for name, t in (("k_pack", k_pack), ("k_params", k_params), ("v_pack", v_pack), ("v_params", v_params)):
@@ -138,7 +144,7 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     `dst_offsets` (int32 [b] device tensor) give the token position, a multiple of 128, at which
     the n new tokens are written, so a full fp16 residual block can be appended to the cache.
     """
-    _check_quant(quant_mode, group_size, num_bits)
+    mode = _check_quant(quant_mode, group_size, num_bits)
     if k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
         raise RuntimeError("k_cache and v_cache must both be [batch, seqlen, nheads_k, head_dim]")
     if not k_cache.is_cuda:
@@ -148,7 +154,7 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     dtype = _dtype_code(k_cache)
     device = k_cache.device
     b, n, h_k, d = k_cache.shape
-    cb, S, ch_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device)
+    cb, S, ch_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device, mode == _lib.K_TENSOR)
     paged = opt_block_table is not None
     if paged:      # the cache tensors are page pools: leading dimension = pages, S = page size
         _check_block_table(opt_block_table, b, device)
@@ -176,6 +182,7 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     a.dst_offset = int(dst_offset)
     a.dst_offsets = None if dst_offsets is None else _i32_dev(dst_offsets, b, device, "dst_offsets").data_ptr()
     a.bits, a.group_size, a.dtype = num_bits, group_size, dtype
+    a.quant_mode = mode
     if paged:
         _set_paging(a, opt_block_table, cb)
     with torch.cuda.device(device):
@@ -228,7 +235,7 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
                          return_lse: bool = False,
                          _stream_ws: bool = False) -> DecodePlan:
     """Validates a decode call and returns a `DecodePlan`; see `fwd_kvcache_int`."""
-    _check_quant(quant_mode, group_size, num_bits)
+    mode = _check_quant(quant_mode, group_size, num_bits)
     if q.dim() != 4 or q.shape[1] != 1:
         raise RuntimeError("q must be [batch, 1, nheads, head_dim] (one query token per sequence)")
     if not q.is_cuda:
@@ -236,7 +243,7 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
     dtype = _dtype_code(q)
     device = q.device
     b, _, h, d = q.shape
-    cb, S, h_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device)
+    cb, S, h_k = _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, device, mode == _lib.K_TENSOR)
     paged = opt_block_table is not None
     if paged:      # page pools: cb pages of S tokens; a sequence holds up to max_pages_per_seq * S tokens
         _check_block_table(opt_block_table, b, device)
@@ -312,6 +319,7 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
         a.softmax_lse = lse.data_ptr()
     a.b, a.h, a.h_k, a.d = b, h, h_k, d
     a.bits, a.group_size, a.dtype = num_bits, group_size, dtype
+    a.quant_mode = mode
     a.softmax_scale = float(softmax_scale)
     L = _lib.lib()
     with torch.cuda.device(device):
@@ -379,6 +387,8 @@ def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: tor
                                 return_lse: bool = False,
                                 _stream_ws: bool = False) -> DecodePlan:
     """Validates a decode step with append and returns its `DecodePlan`; see `fwd_kvcache_int_append`."""
+    if quant_mode == "k-tensor":
+        raise NotImplementedError("the decode step with append is not implemented for quant_mode 'k-tensor'")
     if k_residual is None or v_residual is None or k_residual.dim() != 4 or k_residual.shape[1] < CHUNK:
         raise RuntimeError(f"the residual window must hold at least {CHUNK} tokens")
     max_len = int(max_len)

@@ -109,12 +109,16 @@ def _fp16_bits_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
-def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int, gs: int, dtype: str = "fp16"):
+def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int, gs: int, dtype: str = "fp16",
+                  quant_mode: str = "k-channel"):
     """Logical -> physical.  codes uint8 [b,S,h,128]; k_scale/k_zero uint16 bit patterns of the
     element type `dtype` [b,S/gs,h,128]; v_scale/v_zero uint16 [b,S,h,128/gs].  Returns the four
     cache tensors as numpy arrays with the reference shapes (k_pack/v_pack uint16,
     k_params/v_params float32 containers).  Parameters are stored as fp16 bits for both element
-    types (bf16 values are converted, exact inside the fp16 normal range)."""
+    types (bf16 values are converted, exact inside the fp16 normal range).
+    With quant_mode "k-tensor" k_scale/k_zero are [b,S,h,128/gs] like V's and k_params takes
+    v_params' shape; per chunk its bytes are [64-token half][channel group][16-token tile][token]
+    (scale, zero) pairs, the order in which the decode kernel's score tiles need them."""
     if dtype == "bf16":
         k_scale, k_zero, v_scale, v_zero = (_bf16_bits_to_fp16_bits(np.ascontiguousarray(a))
                                             for a in (k_scale, k_zero, v_scale, v_zero))
@@ -127,9 +131,16 @@ def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int,
     vch = v_codes.reshape(b, nc, CHUNK, h, d).transpose(0, 3, 1, 2, 4)
     k_pack = _codes_to_dwords(kch, kt, kc_, bits).reshape(-1).view(np.uint16).reshape(b, S // pn, h, d)
     v_pack = _codes_to_dwords(vch, vt, vc_, bits).reshape(-1).view(np.uint16).reshape(b, S, h, d // pn)
-    # K params: [b,h,group][scale 128 | zero 128]
-    kp = np.stack([k_scale.transpose(0, 2, 1, 3), k_zero.transpose(0, 2, 1, 3)], axis=3)   # [b,h,G,2,128]
-    k_params = np.ascontiguousarray(kp).astype(np.uint16).reshape(-1).view(np.float32).reshape(b, S // gs, h, d)
+    if quant_mode == "k-tensor":
+        # K params: [b,h,chunk][half][cg][tile][token][scale, zero]
+        ks = k_scale.reshape(b, nc, 2, 4, 16, h, ncg).transpose(0, 5, 1, 2, 6, 3, 4)     # [b,h,nc,half,cg,tile,tok]
+        kz = k_zero.reshape(b, nc, 2, 4, 16, h, ncg).transpose(0, 5, 1, 2, 6, 3, 4)
+        kp = np.stack([ks, kz], axis=-1)
+        k_params = np.ascontiguousarray(kp).astype(np.uint16).reshape(-1).view(np.float32).reshape(b, d // gs, h, S)
+    else:
+        # K params: [b,h,group][scale 128 | zero 128]
+        kp = np.stack([k_scale.transpose(0, 2, 1, 3), k_zero.transpose(0, 2, 1, 3)], axis=3)   # [b,h,G,2,128]
+        k_params = np.ascontiguousarray(kp).astype(np.uint16).reshape(-1).view(np.float32).reshape(b, S // gs, h, d)
     # V params: [b,h,chunk][sb][cg][which][q][i]
     tokmap = v_param_token_map()                                               # [4,4,8]
     vs = v_scale.reshape(b, nc, CHUNK, h, ncg).transpose(0, 3, 1, 4, 2)       # [b,h,nc,cg,128]
@@ -142,7 +153,8 @@ def pack_physical(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, bits: int,
     return k_pack, k_params, v_pack, v_params
 
 
-def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int, dtype: str = "fp16"):
+def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int, dtype: str = "fp16",
+                    quant_mode: str = "k-channel"):
     """Physical -> logical; inverse of pack_physical.  Inputs are numpy arrays with the reference
     shapes (any 16-bit / 32-bit dtype).  Returns (k_codes, k_scale, k_zero, v_codes, v_scale,
     v_zero) with scale/zero as uint16 bit patterns of the element type `dtype`."""
@@ -158,9 +170,15 @@ def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int, dtyp
     vd = np.ascontiguousarray(v_pack).reshape(-1).view(np.uint32).reshape(b, h, nc, ndw)
     k_codes = _dwords_to_codes(kd, kt, kc_, bits).transpose(0, 2, 3, 1, 4).reshape(b, S, h, d)
     v_codes = _dwords_to_codes(vd, vt, vc_, bits).transpose(0, 2, 3, 1, 4).reshape(b, S, h, d)
-    kp = np.ascontiguousarray(k_params).reshape(-1).view(np.uint16).reshape(b, h, S // gs, 2, d)
-    k_scale = np.ascontiguousarray(kp[:, :, :, 0].transpose(0, 2, 1, 3))
-    k_zero = np.ascontiguousarray(kp[:, :, :, 1].transpose(0, 2, 1, 3))
+    if quant_mode == "k-tensor":
+        kp = np.ascontiguousarray(k_params).reshape(-1).view(np.uint16).reshape(b, h, nc, 2, ncg, 4, 16, 2)
+        kp = kp.transpose(0, 2, 3, 5, 6, 1, 4, 7)                                # [b,nc,half,tile,tok,h,cg,2]
+        k_scale = np.ascontiguousarray(kp[..., 0]).reshape(b, S, h, ncg)
+        k_zero = np.ascontiguousarray(kp[..., 1]).reshape(b, S, h, ncg)
+    else:
+        kp = np.ascontiguousarray(k_params).reshape(-1).view(np.uint16).reshape(b, h, S // gs, 2, d)
+        k_scale = np.ascontiguousarray(kp[:, :, :, 0].transpose(0, 2, 1, 3))
+        k_zero = np.ascontiguousarray(kp[:, :, :, 1].transpose(0, 2, 1, 3))
     vp = np.ascontiguousarray(v_params).reshape(-1).view(np.uint16).reshape(b, h, nc, 4, ncg, 2, 4, 8)
     tokmap = v_param_token_map()
     vs = np.zeros((b, h, nc, ncg, CHUNK), np.uint16)
@@ -172,3 +190,65 @@ def unpack_physical(k_pack, k_params, v_pack, v_params, bits: int, gs: int, dtyp
     if dtype == "bf16":
         k_scale, k_zero, v_scale, v_zero = (_fp16_bits_to_bf16_bits(a) for a in (k_scale, k_zero, v_scale, v_zero))
     return k_codes, k_scale, k_zero, v_codes, v_scale, v_zero
+
+
+# --------------------------------------------------------------------------------------------------
+# The reference's own physical layout (4 bits, group size 128, "k-channel"), as far as it can be derived
+# from its sources: the word packing of its quantizer (csrc/bit_decode/src/include/qpack.h:259-294), the
+# consumer's nibble-to-column rule (include/dequantize.h:352-375) and the parameter stores
+# (src/flash_fwd_kernel.h:939-964).  A cache packed by the reference's CUDA kernels could not be produced
+# here, so these converters are pinned by round trips and a hand-built example only: parity with a real
+# CUDA cache is unpinned.
+#   k_pack   [b, S/4, h, 128] u16: row 32*B + p, channel c holds tokens 128*B + p + 32*t in nibble t
+#   k_params [b, S/128, h, 128] f32 = 256 halves per (group, head): scale[c] (128) | zero[c] (128)
+#   v_pack   [b, S, h, 32] u16: token n, column pc holds channels pc + 32*t in nibble t
+#   v_params [b, 1, h, S] f32 = per head and 128-token block 256 halves: scale[n] (128) | zero[n] (128)
+# --------------------------------------------------------------------------------------------------
+def to_reference_layout(k_codes, k_scale, k_zero, v_codes, v_scale, v_zero):
+    """Logical form (4 bits, group size 128; scale/zero as uint16 fp16 bit patterns) -> the four
+    tensors in the reference's layout."""
+    b, S, h, d = k_codes.shape
+    assert d == D and S % CHUNK == 0 and k_scale.shape == (b, S // 128, h, d) and v_scale.shape == (b, S, h, 1)
+    nb = S // 128
+    sh = (np.arange(4, dtype=np.uint16) * 4)
+    kc = k_codes.reshape(b, nb, 4, 32, h, d).astype(np.uint16)                  # token = 128*B + 32*t + p
+    k_pack = (kc << sh[None, None, :, None, None, None]).sum(axis=2, dtype=np.uint16).reshape(b, S // 4, h, d)
+    vc = v_codes.reshape(b, S, h, 4, 32).astype(np.uint16)                      # channel = 32*t + pc
+    v_pack = (vc << sh[None, None, None, :, None]).sum(axis=3, dtype=np.uint16)
+    kp = np.concatenate([k_scale, k_zero], axis=3).astype(np.uint16)            # [b, G, h, 256]
+    k_params = np.ascontiguousarray(kp).reshape(-1).view(np.float32).reshape(b, nb, h, d)
+    vs = v_scale[..., 0].reshape(b, nb, 128, h).transpose(0, 3, 1, 2)           # [b, h, B, 128]
+    vz = v_zero[..., 0].reshape(b, nb, 128, h).transpose(0, 3, 1, 2)
+    vp = np.concatenate([vs, vz], axis=3).astype(np.uint16)                     # [b, h, B, 256]
+    v_params = np.ascontiguousarray(vp).reshape(-1).view(np.float32).reshape(b, h, 1, S).transpose(0, 2, 1, 3)
+    return k_pack, k_params, v_pack, np.ascontiguousarray(v_params)
+
+
+def from_reference_layout(k_pack, k_params, v_pack, v_params):
+    """Inverse of to_reference_layout."""
+    b, S, h, pc = v_pack.shape
+    assert pc == 32 and S % CHUNK == 0
+    nb = S // 128
+    sh = (np.arange(4, dtype=np.uint16) * 4)
+    kw = np.ascontiguousarray(k_pack).view(np.uint16).reshape(b, nb, 1, 32, h, D)
+    k_codes = ((kw >> sh[None, None, :, None, None, None]) & 0xF).astype(np.uint8).reshape(b, S, h, D)
+    vw = np.ascontiguousarray(v_pack).view(np.uint16).reshape(b, S, h, 1, 32)
+    v_codes = ((vw >> sh[None, None, None, :, None]) & 0xF).astype(np.uint8).reshape(b, S, h, D)
+    kp = np.ascontiguousarray(k_params).reshape(-1).view(np.uint16).reshape(b, nb, h, 256)
+    k_scale, k_zero = np.ascontiguousarray(kp[..., :128]), np.ascontiguousarray(kp[..., 128:])
+    vp = np.ascontiguousarray(np.ascontiguousarray(v_params).transpose(0, 2, 1, 3)).reshape(-1).view(np.uint16)
+    vp = vp.reshape(b, h, nb, 256)
+    v_scale = np.ascontiguousarray(vp[..., :128].transpose(0, 2, 3, 1)).reshape(b, S, h, 1)
+    v_zero = np.ascontiguousarray(vp[..., 128:].transpose(0, 2, 3, 1)).reshape(b, S, h, 1)
+    return k_codes, k_scale, k_zero, v_codes, v_scale, v_zero
+
+
+def import_reference_cache(k_pack, k_params, v_pack, v_params):
+    """A 4-bit, group-128 cache in the reference's layout -> the same cache in this library's layout
+    (same tensor shapes)."""
+    return pack_physical(*from_reference_layout(k_pack, k_params, v_pack, v_params), 4, 128)
+
+
+def export_reference_cache(k_pack, k_params, v_pack, v_params):
+    """This library's 4-bit, group-128 cache -> the reference's layout."""
+    return to_reference_layout(*unpack_physical(k_pack, k_params, v_pack, v_params, 4, 128))

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define BITDECODE_ABI_VERSION 3
+#define BITDECODE_ABI_VERSION 4
 
 enum {
     BITDECODE_OK = 0,
@@ -30,6 +30,13 @@ enum {
 };
 
 enum { BITDECODE_FP16 = 0, BITDECODE_BF16 = 1 };
+
+/* quant_mode of the reference's entry points (bit_decode_interface.py:17,50): K quantized per channel over
+ * groups of tokens ("k-channel"), or per token over groups of channels like V ("k-tensor":
+ * csrc/bit_decode/src/include/qpack.h:378-470, dequantize.h:403-475; its dispatch is commented out in the
+ * reference, decode_api.cpp:195-203, 217-225).  "k-tensor" is implemented for 4 bits, as in the reference,
+ * and not for bitdecode_fwd_append; k_params then has v_params' shape. */
+enum { BITDECODE_K_CHANNEL = 0, BITDECODE_K_TENSOR = 1 };
 
 /* Quantize-pack n_tokens new tokens of K and V into the packed cache.
  * Replaces kvcache_qpack<num_bits> (csrc/bit_decode/decode_api.cpp:517-603) and the kernel it
@@ -63,6 +70,7 @@ typedef struct bitdecode_qpack_args {
     int64_t block_table_stride;/* elements between the rows of two sequences                */
     int32_t max_pages_per_seq; /* columns of block_table                                    */
     int32_t num_pages;         /* pages in the pool (leading dimension of the cache)        */
+    int32_t quant_mode;        /* BITDECODE_K_CHANNEL / BITDECODE_K_TENSOR                  */
 } bitdecode_qpack_args;
 
 int bitdecode_qpack(const bitdecode_qpack_args* args, void* stream);
@@ -107,6 +115,7 @@ typedef struct bitdecode_fwd_args {
     int64_t block_table_stride;
     int32_t max_pages_per_seq;
     int32_t num_pages;
+    int32_t quant_mode;        /* BITDECODE_K_CHANNEL / BITDECODE_K_TENSOR                  */
 } bitdecode_fwd_args;
 
 int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);

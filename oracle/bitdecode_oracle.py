@@ -25,6 +25,8 @@ dequantize_ref  : pinned (exactness on an exact grid, error bound scale/2 agains
 attend_ref      : pinned (reduces to softmax(QK^T)V; block-order invariance).
 lse_combine_ref : pinned (closed form, split-count invariance).
 num_splits_heuristic_ref : pinned (known answers from the reference's own comment).
+"k-tensor" mode : quantize_kv_ref / dequantize_ref with K grouped like V; pinned by the same closed
+    forms and one-hot axis probes (tests/test_oracle.py); no C witness for this mode.
 bf16 variants   : the reference has no bf16 kernel; "parity unpinned" by any
     reference artefact, pinned only by the same invariants as fp16.
 """
@@ -124,12 +126,20 @@ class QuantKV:
     v_codes: np.ndarray   # uint8 [b, S, h_k, d]
     v_scale: np.ndarray   # fp32  [b, S, h_k, d/gs]
     v_zero: np.ndarray    # fp32  [b, S, h_k, d/gs]
+    quant_mode: str = "k-channel"   # "k-tensor": k_scale / k_zero are [b, S, h_k, d/gs] like V's
 
 
 def quantize_kv_ref(k: np.ndarray, v: np.ndarray, bits: int, group_size: int,
-                    dtype: str = "fp16") -> QuantKV:
+                    dtype: str = "fp16", quant_mode: str = "k-channel") -> QuantKV:
     """K per-channel (groups of `group_size` consecutive tokens of one channel),
     V per-token (groups of `group_size` consecutive channels of one token).
+
+    quant_mode "k-tensor" (qpack.h:378-470, quant_Ktensor; its dispatch is commented out in the
+    reference, decode_api.cpp:195-203, 217-225): K is quantized like V, per token over groups of
+    `group_size` consecutive channels -- the reduction runs over the fragment's channel index and the
+    four lanes of a quad (qpack.h:313-375: thread_reduce_g over size<1>/num_params columns, then
+    quad_allreduce_g), i.e. over channels of one token; same arithmetic (qpack.h:398-411, 424-449).
+    The reference has it for 4 bits only (qpack.h:385).
 
     Grouping axes: the K operand is reduced over the token index of the MMA fragment and
     the V operand over its channel index (qpack.h:11-84 applied at
@@ -143,13 +153,18 @@ def quantize_kv_ref(k: np.ndarray, v: np.ndarray, bits: int, group_size: int,
     gs = group_size
     if S % gs or d % gs:
         raise ValueError("S and d must be multiples of group_size")
-    kg = k.reshape(b, S // gs, gs, h, d)
-    kc, ks, kz = quantize_group(kg, bits, axis=2, dtype=dtype)
+    if quant_mode not in ("k-channel", "k-tensor"):
+        raise ValueError(quant_mode)
     vg = v.reshape(b, S, h, d // gs, gs)
     vc, vs, vz = quantize_group(vg, bits, axis=4, dtype=dtype)
-    return QuantKV(bits, gs, dtype,
-                   kc.reshape(b, S, h, d), ks[:, :, 0], kz[:, :, 0],
-                   vc.reshape(b, S, h, d), vs[..., 0], vz[..., 0])
+    if quant_mode == "k-tensor":
+        kc, ks, kz = quantize_group(k.reshape(b, S, h, d // gs, gs), bits, axis=4, dtype=dtype)
+        ks, kz = ks[..., 0], kz[..., 0]
+    else:
+        kc, ks, kz = quantize_group(k.reshape(b, S // gs, gs, h, d), bits, axis=2, dtype=dtype)
+        ks, kz = ks[:, :, 0], kz[:, :, 0]
+    return QuantKV(bits, gs, dtype, kc.reshape(b, S, h, d), ks, kz,
+                   vc.reshape(b, S, h, d), vs[..., 0], vz[..., 0], quant_mode)
 
 
 def dequantize_ref(qkv: QuantKV):
@@ -158,8 +173,9 @@ def dequantize_ref(qkv: QuantKV):
     Returns (k_hat, v_hat) fp32 [b, S, h_k, d]."""
     gs = qkv.group_size
     b, S, h, d = qkv.k_codes.shape
-    ks = np.repeat(qkv.k_scale, gs, axis=1)
-    kz = np.repeat(qkv.k_zero, gs, axis=1)
+    k_axis = 3 if qkv.quant_mode == "k-tensor" else 1      # dequantize.h:403-475 / :291
+    ks = np.repeat(qkv.k_scale, gs, axis=k_axis)
+    kz = np.repeat(qkv.k_zero, gs, axis=k_axis)
     k_hat = qkv.k_codes.astype(F32) * ks + kz
     vs = np.repeat(qkv.v_scale, gs, axis=3)
     vz = np.repeat(qkv.v_zero, gs, axis=3)

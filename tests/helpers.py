@@ -24,13 +24,14 @@ def bits16(x: np.ndarray, dtype: str) -> np.ndarray:
     return (x.view(np.uint32) >> 16).astype(np.uint16)
 
 
-def alloc_cache(b, S, h_k, bits, gs, device, fill=None):
-    """Caller-side allocation with the reference's shapes (evaluation/test.py:74-83)."""
+def alloc_cache(b, S, h_k, bits, gs, device, fill=None, k_tensor=False):
+    """Caller-side allocation with the reference's shapes (evaluation/test.py:74-83); in "k-tensor" mode
+    k_params has v_params' shape."""
     pn = 16 // bits
     d = 128
     mk = torch.zeros if fill is None else (lambda *a, **k: torch.full(*a, fill_value=fill, **k))
     k_pack = mk((b, S // pn, h_k, d), dtype=torch.uint16, device=device)
-    k_params = torch.zeros((b, S // gs, h_k, d), dtype=torch.float32, device=device)
+    k_params = torch.zeros((b, d // gs, h_k, S) if k_tensor else (b, S // gs, h_k, d), dtype=torch.float32, device=device)
     v_pack = mk((b, S, h_k, d // pn), dtype=torch.uint16, device=device)
     v_params = torch.zeros((b, d // gs, h_k, S), dtype=torch.float32, device=device)
     return k_pack, k_params, v_pack, v_params
@@ -57,7 +58,7 @@ def oracle_physical(qkv: O.QuantKV):
     dt = qkv.dtype
     return L.pack_physical(qkv.k_codes, bits16(qkv.k_scale, dt), bits16(qkv.k_zero, dt),
                            qkv.v_codes, bits16(qkv.v_scale, dt), bits16(qkv.v_zero, dt),
-                           qkv.bits, qkv.group_size, dt)
+                           qkv.bits, qkv.group_size, dt, qkv.quant_mode)
 
 
 def assert_cache_equals_oracle(cache_np, qkv: O.QuantKV):
@@ -67,7 +68,7 @@ def assert_cache_equals_oracle(cache_np, qkv: O.QuantKV):
     inside the fp16 normal range)."""
     from bitladder_amd import layout as L
     dt = qkv.dtype
-    kc, ks, kz, vc, vs, vz = L.unpack_physical(*cache_np, qkv.bits, qkv.group_size, "fp16")
+    kc, ks, kz, vc, vs, vz = L.unpack_physical(*cache_np, qkv.bits, qkv.group_size, "fp16", qkv.quant_mode)
     np.testing.assert_array_equal(kc, qkv.k_codes, err_msg="K codes")
     np.testing.assert_array_equal(vc, qkv.v_codes, err_msg="V codes")
 

@@ -36,6 +36,61 @@ def test_layout_roundtrip_and_byte_budget(bits, gs):
         np.testing.assert_array_equal(a, c)
 
 
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_ktensor_layout_roundtrip(gs):
+    """"k-tensor" mode: K parameters per token and channel group, k_params with v_params' shape."""
+    rng = np.random.default_rng(gs)
+    b, S, h, bits, ncg = 2, 256, 3, 4, 128 // gs
+    kc = rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8)
+    vc = rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8)
+    par = [rng.integers(0, 65536, (b, S, h, ncg)).astype(np.uint16) for _ in range(4)]
+    phys = L.pack_physical(kc, par[0], par[1], vc, par[2], par[3], bits, gs, "fp16", "k-tensor")
+    assert phys[1].shape == phys[3].shape == (b, ncg, h, S)
+    back = L.unpack_physical(*phys, bits, gs, "fp16", "k-tensor")
+    for a, c in zip((kc, par[0], par[1], vc, par[2], par[3]), back):
+        np.testing.assert_array_equal(a, c)
+    # the (scale, zero) pair of token n, group g sits at [half][g][tile][token] of its chunk
+    raw = np.ascontiguousarray(phys[1]).reshape(-1).view(np.uint16).reshape(b, h, S // 128, 2, ncg, 4, 16, 2)
+    n, g = 128 + 64 + 16 * 2 + 5, ncg - 1
+    assert raw[1, 2, 1, 1, g, 2, 5, 0] == par[0][1, n, 2, g] and raw[1, 2, 1, 1, g, 2, 5, 1] == par[1][1, n, 2, g]
+
+
+def test_reference_layout_converters_roundtrip_and_hand_built_group():
+    """Converters to and from the reference's own 4-bit, group-128 layout (derived from qpack.h:259-294,
+    dequantize.h:352-375, flash_fwd_kernel.h:939-964).  Pinned by round trips and a hand-built group only:
+    no cache packed by the reference's CUDA kernels exists here (parity with one is unpinned)."""
+    rng = np.random.default_rng(9)
+    b, S, h = 2, 256, 3
+    kc = rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8)
+    vc = rng.integers(0, 16, (b, S, h, 128), dtype=np.uint8)
+    ks, kz = (rng.integers(0, 65536, (b, S // 128, h, 128)).astype(np.uint16) for _ in range(2))
+    vs, vz = (rng.integers(0, 65536, (b, S, h, 1)).astype(np.uint16) for _ in range(2))
+    ref = L.to_reference_layout(kc, ks, kz, vc, vs, vz)
+    # the reference's tensor contract (evaluation/test.py:76-83)
+    assert [a.shape for a in ref] == [(b, S // 4, h, 128), (b, S // 128, h, 128), (b, S, h, 32), (b, 1, h, S)]
+    for a, c in zip((kc, ks, kz, vc, vs, vz), L.from_reference_layout(*ref)):
+        np.testing.assert_array_equal(a, c)
+    ours = L.import_reference_cache(*ref)
+    for a, c in zip(ours, L.pack_physical(kc, ks, kz, vc, vs, vz, 4, 128)):
+        np.testing.assert_array_equal(a, c)
+    for a, c in zip(ref, L.export_reference_cache(*ours)):
+        np.testing.assert_array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(c).view(np.uint8))
+    # by hand: K word of pack row p, channel c = tokens p, p+32, p+64, p+96 of the block in nibbles 0..3;
+    # V word of token n, column pc = channels pc, pc+32, pc+64, pc+96 in nibbles 0..3
+    k_pack, k_params, v_pack, v_params = ref
+    p_, c_ = 7, 19
+    want = sum(int(kc[1, 128 + p_ + 32 * t, 2, c_]) << (4 * t) for t in range(4))
+    assert int(k_pack.view(np.uint16)[1, 32 + p_, 2, c_]) == want
+    n_, pc = 200, 5
+    want = sum(int(vc[0, n_, 1, pc + 32 * t]) << (4 * t) for t in range(4))
+    assert int(v_pack.view(np.uint16)[0, n_, 1, pc]) == want
+    # parameters: 256 halves per (group, head): scale[c] then zero[c]; per 128-token block: scale[n] then zero[n]
+    kh = np.ascontiguousarray(k_params).view(np.uint16).reshape(b, S // 128, h, 256)
+    assert kh[1, 1, 2, c_] == ks[1, 1, 2, c_] and kh[1, 1, 2, 128 + c_] == kz[1, 1, 2, c_]
+    vh = np.ascontiguousarray(v_params[:, 0]).view(np.uint16).reshape(b, h, S // 128, 256)
+    assert vh[0, 1, 1, n_ - 128] == vs[0, n_, 1, 0] and vh[0, 1, 1, 128 + n_ - 128] == vz[0, n_, 1, 0]
+
+
 def test_bf16_parameters_are_stored_as_fp16_bits():
     """A bf16 cache keeps scale/zero as fp16 bit patterns: bf16 values inside the fp16 normal range
     survive pack -> unpack unchanged, and the stored pattern is the fp16 encoding of the value."""
@@ -221,8 +276,10 @@ def test_python_entry_points_validate_before_touching_the_gpu():
     from bitladder_amd import fwd_kvcache_int, kvcache_pack_int
     t = torch.zeros(1, 128, 2, 128, dtype=torch.float16)
     kp = torch.zeros(1, 32, 2, 128, dtype=torch.uint16)
-    with pytest.raises(NotImplementedError):
-        kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-tensor", 128, 4)
+    with pytest.raises(NotImplementedError):      # "k-tensor" is a 4-bit mode, as in the reference
+        kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-tensor", 128, 2)
+    with pytest.raises(ValueError):
+        kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-token", 128, 4)
     with pytest.raises(ValueError):
         kvcache_pack_int(t, kp, kp, t, kp, kp, None, None, 128, "k-channel", 48, 4)
     with pytest.raises(ValueError):

@@ -193,6 +193,42 @@ def test_dequantize_axes_with_one_hot_parameters():
     np.testing.assert_array_equal(v_hat, want_v)
 
 
+# ------------------------------------------------------------------ "k-tensor" mode
+def test_ktensor_mode_quantizes_k_like_v():
+    """quant_mode "k-tensor" (qpack.h:378-470): K per token over channel groups -- the V quantizer applied to K."""
+    _, k, v = O.make_inputs(2, 2, 2, 128, 0, seed=77)
+    a = O.quantize_kv_ref(k, v, 4, 32, "fp16", "k-tensor")
+    as_v = O.quantize_kv_ref(v, k, 4, 32)             # K in V's place
+    assert a.k_scale.shape == (2, 128, 2, 4)
+    np.testing.assert_array_equal(a.k_codes, as_v.v_codes)
+    np.testing.assert_array_equal(a.k_scale, as_v.v_scale)
+    np.testing.assert_array_equal(a.k_zero, as_v.v_zero)
+    np.testing.assert_array_equal(a.v_codes, O.quantize_kv_ref(k, v, 4, 32).v_codes)     # V is untouched by the mode
+    # hand-computed token: channels 0..31 hold 0, 1, ..., 15, 0, ... -> range 15, scale 1, codes = values
+    k2 = np.zeros((1, 128, 1, 128), F32)
+    k2[0, 5, 0, :16] = np.arange(16)
+    k2[0, 5, 0, 40] = 30.0                            # another channel group of the same token: range 30, scale 2
+    b_ = O.quantize_kv_ref(k2, k2, 4, 32, "fp16", "k-tensor")
+    assert b_.k_codes[0, 5, 0, :16].tolist() == list(range(16)) and b_.k_scale[0, 5, 0, 0] == 1.0
+    assert b_.k_codes[0, 5, 0, 40] == 15 and b_.k_scale[0, 5, 0, 1] == 2.0 and np.count_nonzero(b_.k_scale) == 2
+    k_hat, _ = O.dequantize_ref(b_)
+    np.testing.assert_array_equal(k_hat, k2)
+
+
+def test_ktensor_dequantize_axis_with_one_hot_parameters():
+    b, S, h, d, gs = 1, 128, 1, 128, 32
+    z = lambda *s: np.zeros(s, F32)
+    q = O.QuantKV(4, gs, "fp16", np.ones((b, S, h, d), np.uint8), z(b, S, h, d // gs), z(b, S, h, d // gs),
+                  np.zeros((b, S, h, d), np.uint8), z(b, S, h, d // gs), z(b, S, h, d // gs), "k-tensor")
+    q.k_scale[0, 70, 0, 2] = 3.0        # channel group 2 (channels 64..95) of token 70
+    q.k_zero[0, 9, 0, 0] = -1.0
+    k_hat, _ = O.dequantize_ref(q)
+    want = z(b, S, h, d)
+    want[0, 70, 0, 64:96] = 3.0
+    want[0, 9, 0, 0:32] = -1.0
+    np.testing.assert_array_equal(k_hat, want)
+
+
 # ------------------------------------------------------------------ second witness (C restatement)
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("bits,gs", [(4, 128), (4, 32), (2, 64), (2, 128)])
