@@ -177,6 +177,7 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     P.b = a->b; P.n_tokens = a->n_tokens; P.hk = a->h_k;
     P.dst_offset = a->dst_offset;
     P.dst_offsets = a->dst_offsets;
+    P.capacity = static_cast<int>(std::min<int64_t>(capacity, INT32_MAX / 2));
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
     P.block_table = a->block_table; P.bt_stride = a->block_table_stride;
     P.chunks_per_page = a->cache_tokens / kChunk;
@@ -299,6 +300,11 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     P.block_table = a->block_table; P.bt_stride = a->block_table_stride;
     P.chunks_per_page = a->block_table ? a->cache_tokens / kChunk : 1;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;
+    {
+        const int64_t cap = a->block_table ? static_cast<int64_t>(a->max_pages_per_seq) * a->cache_tokens : a->cache_tokens;
+        P.capacity = static_cast<int>(std::min<int64_t>(cap, INT32_MAX / 2));
+        P.res_cap = max_r;
+    }
     uint8_t* ws = static_cast<uint8_t*>(a->workspace);
     if (step) {
         P.lengths = step->lengths;
@@ -308,8 +314,6 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
         P.v_new = static_cast<const uint16_t*>(step->v_new);
         P.knew_sb = step->knew_stride_b; P.knew_sh = step->knew_stride_h;
         P.vnew_sb = step->vnew_stride_b; P.vnew_sh = step->vnew_stride_h;
-        const int64_t cap = a->block_table ? static_cast<int64_t>(a->max_pages_per_seq) * a->cache_tokens : a->cache_tokens;
-        P.capacity = static_cast<int>(std::min<int64_t>(cap, INT32_MAX / 2));
     }
     if (nsplit > 1 && static_scratch) {
         P.tickets = reinterpret_cast<int*>(static_scratch);

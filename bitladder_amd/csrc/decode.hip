@@ -90,8 +90,10 @@ __device__ unsigned long long* g_prof = nullptr;
 #define PROF_FLUSH() do { } while (0)
 #endif
 
-constexpr float kPShift = 2.0f;   // probabilities are kept as 2^kPShift * exp2(s - max): a V scale
-                                  // is at most 65504*2/3, so p*scale cannot overflow fp16
+// Probabilities are kept as 2^shift * exp2(s - max) in fp16, and p * (V scale) must stay inside the fp16
+// range as well.  A 4-bit V scale is at most 131008 / 15 = 8734: p up to 4 is safe and keeps two more bits of
+// the small probabilities.  A 2-bit V scale reaches 131008 / 3 = 43669: p stays at 1 or below.
+constexpr float p_shift(int bits) { return bits == 4 ? 2.0f : 0.0f; }
 constexpr int kLdsRowHalves = 136;
 
 __device__ __forceinline__ h2 pk_rtz(float a, float b) {
@@ -202,11 +204,11 @@ struct WaveState {
 };
 
 // Online-softmax step over N raw scores t (q.k units); on return t holds
-// p = 2^kPShift * exp2(scale * (t - running max)).  Accumulators are rescaled only when the
+// p = 2^pshift * exp2(scale * (t - running max)).  Accumulators are rescaled only when the
 // running max of some head moved (wave-uniform branch).  With HALVES the hi column and the lo
 // column of a head hold different halves of the step's scores, and the maximum is taken over both.
 template <int N, int NCG, bool HALVES = false>
-__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st, float mx) {
+__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st, float mx, float pshift) {
     if constexpr (HALVES) mx = fmaxf(mx, partner(mx));
     mx = colmax(mx);
     const float m_new = fmaxf(st.m, mx);
@@ -220,16 +222,16 @@ __device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveSta
         for (int ct = 0; ct < 8; ++ct) st.o[ct] *= alpha;
         st.m = m_new;
     }
-    const float c0 = kPShift - m_use * scale;
+    const float c0 = pshift - m_use * scale;
 #pragma unroll
     for (int i = 0; i < N; ++i) t[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(t[i], scale, c0));
 }
 template <int N, int NCG>
-__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st) {
+__device__ __forceinline__ void softmax_step(float (&t)[N], float scale, WaveState<NCG>& st, float pshift) {
     float mx = t[0];
 #pragma unroll
     for (int i = 1; i < N; ++i) mx = fmaxf(mx, t[i]);
-    softmax_step<N, NCG>(t, scale, st, mx);
+    softmax_step<N, NCG>(t, scale, st, mx, pshift);
 }
 
 // Accumulators of the four S^T tiles of a 64-token step -> probabilities as operands of the second
@@ -248,7 +250,7 @@ __device__ __forceinline__ void step_probabilities(const f4 (&sc)[4], uint32_t h
 #pragma unroll
         for (int r = 0; r < 4; ++r) t[4 * tt + r] = sc[tt][r] + partner(sc[tt][r]);
     }
-    softmax_step<16, NCG>(t, scale, st);
+    softmax_step<16, NCG>(t, scale, st, p_shift(4));
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         u4 pw;
@@ -293,7 +295,7 @@ __device__ __forceinline__ void step_probabilities_shared(const f4 (&sc)[4], uin
                    "=&v"(mx)
                  : "v"(sc[2][0]), "v"(sc[2][1]), "v"(sc[2][2]), "v"(sc[2][3]), "v"(sc[3][0]), "v"(sc[3][1]),
                    "v"(sc[3][2]), "v"(sc[3][3]));
-    softmax_step<8, NCG, true>(t, scale, st, mx);
+    softmax_step<8, NCG, true>(t, scale, st, mx, p_shift(2));
     u4 pw;
 #pragma unroll
     for (int x = 0; x < 4; ++x) pw[x] = __builtin_bit_cast(uint32_t, pk_rtz(t[2 * x], t[2 * x + 1]));
@@ -950,7 +952,7 @@ __device__ __forceinline__ void load_fp16_tile(Fp16Tile& T, const WindowSrc& W, 
 
 template <bool BF16, int NCG>
 __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P, int n0, int R, int lane,
-                                          const QRows& Q, bool lo_part, WaveState<NCG>& st, uint16_t* lds) {
+                                          const QRows& Q, bool lo_part, WaveState<NCG>& st, uint16_t* lds, float pshift) {
     const int col = lane & 15, kg = lane >> 4;
 
     // V tile (16 tokens x 128 channels) goes through this wave's LDS slab to be read back
@@ -977,7 +979,7 @@ __device__ __forceinline__ void fp16_tile(const Fp16Tile& T, const FwdParams& P,
             s[r] = tk < R ? tot : -INFINITY;
         }
     }
-    softmax_step<4, NCG>(s, P.scale_log2, st);
+    softmax_step<4, NCG>(s, P.scale_log2, st, pshift);
     const h2 p01 = pk_rtz(s[0], s[1]), p23 = pk_rtz(s[2], s[3]);
     h4 pb = {p01[0], p01[1], p23[0], p23[1]};
     if (lo_part) pb = h4{0, 0, 0, 0};
@@ -1116,7 +1118,8 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 // Final values of one query head: lane l writes channels 2l, 2l+1 of O / L, lane 0 the natural-log LSE
 // (softmax.h:303; +inf for a row without keys).
 template <bool BF16>
-__device__ __forceinline__ void write_head(uint16_t* out_row, float* lse, int lane, float O0, float O1, float M, float L) {
+__device__ __forceinline__ void write_head(uint16_t* out_row, float* lse, int lane, float O0, float O1, float M, float L,
+                                           float pshift) {
     const bool none = !(L > 0.0f);
     const uint16_t a = to_out<BF16>(none ? 0.0f : O0 / L), b = to_out<BF16>(none ? 0.0f : O1 / L);
     if ((reinterpret_cast<uintptr_t>(out_row) & 3u) == 0) {
@@ -1125,7 +1128,7 @@ __device__ __forceinline__ void write_head(uint16_t* out_row, float* lse, int la
         out_row[2 * lane] = a;
         out_row[2 * lane + 1] = b;
     }
-    if (lane == 0 && lse) *lse = none ? INFINITY : (M + __log2f(L) - kPShift) * 0.69314718055994531f;
+    if (lane == 0 && lse) *lse = none ? INFINITY : (M + __log2f(L) - pshift) * 0.69314718055994531f;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1273,8 +1276,9 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         S = min(step_len - r_new, P.capacity);     // a length beyond the capacity is the caller's error: stay inside
         R = r_new + 1;
     } else {
-        S = P.seqlens ? P.seqlens[bi] : P.seqlen;
-        R = P.reslens ? P.reslens[bi] : P.reslen;
+        // per-sequence values are device data the host never saw: keep them inside the cache and the window
+        S = P.seqlens ? min(max(P.seqlens[bi], 0), P.capacity) : P.seqlen;
+        R = P.reslens ? min(max(P.reslens[bi], 0), P.res_cap) : P.reslen;
     }
     const int nU = (S / kChunk) * C::UPC;
     const int ups = (nU + P.nsplit - 1) / P.nsplit;
@@ -1366,7 +1370,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
             while (true) {
                 const int tn = t + stride;
                 const bool more = tn < nT;
-                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, Q, lo_part, st, slab);
+                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, Q, lo_part, st, slab, p_shift(BITS));
                 if (!more) break;
                 load_fp16_tile<APPEND>(T, W, tn * 16, R, lane, r_new);
                 t = tn;
@@ -1462,7 +1466,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
             O1 = __builtin_fmaf(a, v.y, O1);
         }
         if (P.nsplit == 1) {
-            write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
+            write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
         } else {
             st_dev2(&o_part[(split * hstride + hrow) * kHeadDim + 2 * lane], O0, O1);
             if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M, L);
@@ -1478,7 +1482,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
                 if (wave == 0) *s_last = last;
             } else if (last) {
                 merge_splits(o_part, ml_part, hrow, static_cast<uint32_t>(hstride) * kHeadDim, P.nsplit, lane, O0, O1, M, L);
-                write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
+                write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }
     }
@@ -1493,7 +1497,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
             if (appends) step_begin<NW>(bi, hk, step_len);
             if (wave < g && last) {
                 merge_splits(o_part, ml_part, hrow, static_cast<uint32_t>(hstride) * kHeadDim, P.nsplit, lane, O0, O1, M, L);
-                write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L);
+                write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }
         if (appends) step_end<BITS, GS, BF16>(lds, bi, hk, step_len);

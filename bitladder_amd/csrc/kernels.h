@@ -22,6 +22,7 @@ struct QpackParams {
     int b, n_tokens, hk;
     int dst_offset;
     const int* dst_offsets;
+    int capacity;               // tokens a sequence can hold: a device-side offset beyond it skips the sequence
     int bits, gs, bf16;
     int ktensor;                // "k-tensor" mode: K quantized per token over channel groups, like V
     const int* block_table;     // paged cache: page of (sequence, page slot); regions are then (page, kv-head)
@@ -69,7 +70,8 @@ struct FwdParams {
     const uint16_t* k_new;
     const uint16_t* v_new;
     int64_t knew_sb, knew_sh, vnew_sb, vnew_sh;
-    int capacity;               // packed tokens a sequence can hold
+    int capacity;               // packed tokens a sequence can hold (set for every call; clamps device-side lengths)
+    int res_cap;                // rows of the fp16 window (clamps device-side window lengths)
 };
 
 hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);

@@ -20,6 +20,8 @@ __global__ __launch_bounds__(qp::kPackThreads) void qpack_kernel(QpackParams P) 
     const int dst_base = P.dst_offsets ? P.dst_offsets[bi] : P.dst_offset;
     if (dst_base < 0) return;       // a negative per-sequence offset skips that sequence (whole workgroup)
     const int dst_tok = dst_base + ci_src * kChunk;
+    // a device-side offset the host never saw: not on a chunk boundary, or past the cache -> nothing is written
+    if ((dst_base & (kChunk - 1)) != 0 || dst_tok + kChunk > P.capacity) return;
     const ChunkPlace place = chunk_place(P.block_table, P.bt_stride, P.chunks_per_page, bi, hk, P.hk, dst_tok / kChunk);
     const qp::ChunkDst D = qp::chunk_dst<BITS, GS, KT>(P.k_pack, P.k_params, P.v_pack, P.v_params, P.kpack_bh, P.kparams_bh,
                                                    P.vpack_bh, P.vparams_bh, place);

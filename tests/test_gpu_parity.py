@@ -285,3 +285,56 @@ def test_waves_with_many_units_on_cache_resident_data_are_deterministic(device, 
     k_hat, v_hat = O.dequantize_ref(qkv)
     ref, _ = O.attend_ref(q, k_hat, v_hat, SCALE)
     assert np.abs(outs[0].float().cpu().numpy() - ref).max() < 2e-3
+
+
+@pytest.mark.parametrize("bits,vmax", [(2, 30000.0), (4, 30000.0), (2, 65000.0)])
+def test_decode_with_v_groups_spanning_the_fp16_range(device, bits, vmax):
+    """V groups whose range is close to the whole fp16 range: the V scale reaches 2 * vmax / (2^bits - 1)
+    (43 000 at 2 bits), and probability x scale must still fit fp16."""
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, S, gs = 1, 8, 2, 512, 128
+    q, k, v = O.make_inputs(b, h, h_k, S, 0, seed=61)
+    rng = np.random.default_rng(3)
+    v = O.round_to_storage((rng.uniform(-1, 1, v.shape) * vmax).astype(np.float32), "fp16")
+    v[0, ::7, 0, 5], v[0, ::7, 0, 6] = vmax, -vmax
+    v = O.round_to_storage(v, "fp16")
+    qkv = O.quantize_kv_ref(k, v, bits, gs)
+    assert qkv.v_scale.max() > (1.9 * vmax) / ((1 << bits) - 1)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, _ = O.attend_ref(q, k_hat, v_hat, SCALE)
+    out = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits).float().cpu().numpy()
+    assert np.isfinite(out).all()
+    # outputs are of the order of vmax / sqrt(S): the bound is relative here (2e-3 of the largest expected value)
+    assert np.abs(out - want).max() < 2e-3 * np.abs(want).max(), (np.abs(out - want).max(), np.abs(want).max())
+
+
+def test_device_side_lengths_and_offsets_beyond_the_buffers_are_clamped(device):
+    """Per-sequence lengths and offsets are device data the host never sees: a packed length beyond the cache
+    counts as the capacity, a window length beyond the window as the window, and a pack offset that is off a
+    chunk boundary or past the cache writes nothing."""
+    from bitladder_amd import fwd_kvcache_int, kvcache_pack_int
+    b, h, h_k, S, R, bits, gs = 2, 8, 2, 1024, 64, 4, 128
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=62)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    kr, vr = H.to_dev(k[:, S:], "fp16", device), H.to_dev(v[:, S:], "fp16", device)
+    qd = H.to_dev(q, "fp16", device)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    kw = dict(k_residual=kr, v_residual=vr, max_seqlen_k=S, max_residual_len=R)
+    want = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, seqlens_k=i32([S, 512]), residual_len=i32([R, 10]), **kw)
+    got = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, seqlens_k=i32([S + 4096, 512]),
+                          residual_len=i32([R + 1000, 10]), **kw)
+    assert torch.equal(got, want)
+    neg = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, seqlens_k=i32([S, -128]), residual_len=i32([R, 10]), **kw)
+    zero = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, seqlens_k=i32([S, 0]), residual_len=i32([R, 10]), **kw)
+    assert torch.equal(neg, zero)
+    # pack: sequence 0 at a valid offset, sequence 1 once misaligned and once past the end -> untouched
+    before = [t.clone() for t in cache]
+    kd, vd = H.to_dev(k[:, :128] * 0.5, "fp16", device), H.to_dev(v[:, :128] * 0.5, "fp16", device)
+    for bad in (64, S):
+        kvcache_pack_int(kd, cache[0], cache[1], vd, cache[2], cache[3], None, None, 128, "k-channel", gs, bits,
+                         dst_offsets=i32([256, bad]))
+        torch.cuda.synchronize()
+        for t, t0 in zip(cache, before):
+            assert torch.equal(t[1], t0[1])                  # sequence 1: nothing written
+        assert not torch.equal(cache[0][0], before[0][0])    # sequence 0: its chunk was packed
