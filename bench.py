@@ -171,6 +171,8 @@ def main():
     ap.add_argument("--no-fp16", action="store_true", help="skip the fp16-KV baseline leg")
     ap.add_argument("--no-qpack", action="store_true", help="skip the quantize-pack kernel leg")
     ap.add_argument("--no-step", action="store_true", help="skip the decode-step-with-append leg")
+    ap.add_argument("--no-dropin", action="store_true", help="skip the eager drop-in call leg")
+    ap.add_argument("--no-probe", action="store_true", help="skip the read-probe leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three plain 256 MiB device copies (a kernel of known traffic, used to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -284,28 +286,29 @@ def main():
     if getattr(time_steps, "last_quantiles", None):
         result["us_per_step_quantiles"] = time_steps.last_quantiles
 
-    # what the memory system alone allows: a kernel that only reads as many bytes as one step streams
-    # (same launch shape, buffers rotated like the caches), timed the same way
-    import ctypes
-    from bitladder_amd import _lib
-    L = _lib.lib()
-    probe_bytes = (total_bytes + 4095) // 4096 * 4096
-    probe_bufs = [torch.randint(0, 255, (probe_bytes,), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
+    if not args.no_probe:
+        # what the memory system alone allows: a kernel that only reads as many bytes as one step streams
+        # (same launch shape, buffers rotated like the caches), timed the same way
+        import ctypes
+        from bitladder_amd import _lib
+        L = _lib.lib()
+        probe_bytes = (total_bytes + 4095) // 4096 * 4096
+        probe_bufs = [torch.randint(0, 255, (probe_bytes,), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
 
-    def probe(i):
-        buf = probe_bufs[i % nbuf]
-        _lib.check(L.bitdecode_read_probe(buf.data_ptr(), probe_bytes, None, torch.cuda.current_stream(dev).cuda_stream))
+        def probe(i):
+            buf = probe_bufs[i % nbuf]
+            _lib.check(L.bitdecode_read_probe(buf.data_ptr(), probe_bytes, None, torch.cuda.current_stream(dev).cuda_stream))
 
-    _, epr, _ = time_steps(probe, args.steps, args.warmup, not args.no_graph, replays=replays)
-    us_probe = epr / (args.steps * replays) * 1e6
-    result["roofline"]["read_kernel_us"] = round(us_probe, 3)
-    result["roofline"]["read_kernel_GBs"] = round(probe_bytes / (us_probe * 1e-6) / 1e9, 1)
-    result["roofline"]["frac_of_read_kernel"] = round(us_probe / us_step_ev, 4)
-    del probe_bufs
+        _, epr, _ = time_steps(probe, args.steps, args.warmup, not args.no_graph, replays=replays)
+        us_probe = epr / (args.steps * replays) * 1e6
+        result["roofline"]["read_kernel_us"] = round(us_probe, 3)
+        result["roofline"]["read_kernel_GBs"] = round(probe_bytes / (us_probe * 1e-6) / 1e9, 1)
+        result["roofline"]["frac_of_read_kernel"] = round(us_probe / us_step_ev, 4)
+        del probe_bufs
 
     # the call a user of the reference makes: plain fwd_kvcache_int(...), eager launches, workspace from the
     # per-stream cache (nothing allocated or filled after the first call), output buffer passed in
-    if not ragged:
+    if not ragged and not args.no_dropin:
         from bitladder_amd import fwd_kvcache_int
         outs = [torch.empty_like(plans[i].out) for i in range(nbuf)]
 

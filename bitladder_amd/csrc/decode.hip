@@ -75,16 +75,7 @@ __device__ unsigned long long* g_prof = nullptr;
             for (int i_ = 0; i_ < 16; ++i_) pb[i_] = prof_ts[i_];                                     \
         }                                                                                             \
     } while (0)
-#define PHASE(slot)                                                 \
-    do {                                                            \
-        if (phase_ts) {                                             \
-            __builtin_amdgcn_sched_barrier(0);                      \
-            phase_ts[slot] = __builtin_readcyclecounter();          \
-            __builtin_amdgcn_sched_barrier(0);                      \
-        }                                                           \
-    } while (0)
 #else
-#define PHASE(slot) do { } while (0)
 #define PROF_DECL do { } while (0)
 #define PROF(slot) do { } while (0)
 #define PROF_FLUSH() do { } while (0)
