@@ -24,15 +24,15 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the split-KV kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/fwd_splitkv_and_qpack_llama3-8b-gqa-32k-4bit-g128.md): the counters read 18089.2 and
-# 592.25 per dispatch; a 256 MiB device copy in the same runs reads 131085 and 262144, i.e. the fetch
-# counter is in units of 2 KiB and the write counter in KiB.
+# (profiles/fwd_splitkv_hbm_traffic_all_workloads.md): mean counter values per dispatch at the default split
+# count; a 256 MiB device copy in the same runs reads 131085 and 262144, i.e. the fetch counter is in units of
+# 2 KiB and the write counter in KiB.
 MEASURED_TRAFFIC_BYTES = {
-    "llama3-8b-gqa-32k-4bit-g128": int(18089.2 * 2048 + 592.25 * 1024),
-    # the other workloads, same method (profiles/fwd_splitkv_hbm_traffic_all_workloads.md)
-    "llama2-7b-mha-4k-4bit-g128": int(9955.41 * 2048 + 161.0 * 1024),
-    "llama3-8b-gqa-128k-2bit-g64": int(41731.14 * 2048 + 592.25 * 1024),
-    "llama3-70b-gqa-64k-2bit-g128-b8": int(150316.26 * 2048 + 1290.0 * 1024),
+    "llama3-8b-gqa-32k-4bit-g128": int(18054.07 * 2048 + 585.0 * 1024),
+    "llama2-7b-mha-4k-4bit-g128": int(9924.05 * 2048 + 153.0 * 1024),
+    "llama3-8b-gqa-128k-2bit-g64": int(41682.54 * 2048 + 585.0 * 1024),
+    "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": int(55984.51 * 2048 + 720.0 * 1024),
+    "llama3-70b-gqa-64k-2bit-g128-b8": int(150275.70 * 2048 + 1296.0 * 1024),
 }
 
 WORKLOADS = {
