@@ -13,6 +13,7 @@ import torch
 from . import _lib
 
 _PACK_DTYPES = (torch.uint16, torch.int16)
+_PARAM_DTYPES = (torch.float32,)
 CHUNK = 128
 
 
@@ -72,29 +73,48 @@ def _check_cache(k_pack, k_params, v_pack, v_params, num_bits, group_size, devic
         raise RuntimeError(f"head dimension {d} is not supported (only 128)")
     if S % CHUNK:
         raise RuntimeError(f"packed cache capacity {S} must be a multiple of {CHUNK} tokens")
-    want = {
-        "k_pack": (b, S // pn, h_k, d),
-        "k_params": (b, d // group_size, h_k, S) if k_tensor else (b, S // group_size, h_k, d),
-        "v_pack": (b, S, h_k, d // pn), "v_params": (b, d // group_size, h_k, S),
-    }
-    for name, t in (("k_pack", k_pack), ("k_params", k_params), ("v_pack", v_pack), ("v_params", v_params)):
-        if tuple(t.shape) != want[name]:
-            raise RuntimeError(f"{name} must have shape {want[name]}, got {tuple(t.shape)}")
+    k_params_shape = (b, d // group_size, h_k, S) if k_tensor else (b, S // group_size, h_k, d)
+    for name, t, want, dtypes in (("k_pack", k_pack, (b, S // pn, h_k, d), _PACK_DTYPES),
+                                  ("k_params", k_params, k_params_shape, _PARAM_DTYPES),
+                                  ("v_pack", v_pack, (b, S, h_k, dp), _PACK_DTYPES),
+                                  ("v_params", v_params, (b, d // group_size, h_k, S), _PARAM_DTYPES)):
+        if t.shape != want:
+            raise RuntimeError(f"{name} must have shape {want}, got {tuple(t.shape)}")
         if t.device != device:
             raise RuntimeError(f"{name} must be on {device}")
         if not t.is_contiguous():
             raise RuntimeError(f"{name} must be contiguous")
-    for name, t in (("k_pack", k_pack), ("v_pack", v_pack)):
-        if t.dtype not in _PACK_DTYPES:
-            raise RuntimeError(f"{name} must have dtype torch.uint16")
-    for name, t in (("k_params", k_params), ("v_params", v_params)):
-        if t.dtype != torch.float32:
+        if t.dtype not in dtypes:
+            if dtypes is _PACK_DTYPES:
+                raise RuntimeError(f"{name} must have dtype torch.uint16")
             raise RuntimeError(f"{name} must have dtype torch.float32 (each element holds two 16-bit values)")
     return b, S, h_k
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(device) -> int:
+    """Handle of torch's current stream on `device` (hipStream_t as an integer)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """`with _on_device(device):` makes `device` current for the block; free when it already is."""
+
+    def __init__(self, device):
+        self._ctx = None if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            self._ctx.__exit__(*exc)
+        return False
 
 
 # Split workspaces of the plain entry points, one per (device, stream, kind, batch, heads, splits): a call
@@ -115,6 +135,24 @@ def _stream_workspace(device, kind: str, b: int, h: int, ns: int, nbytes: int) -
         ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
         _WORKSPACES[key] = ws
     return ws
+
+
+_SPLIT_PLANS: "dict[tuple, tuple]" = {}
+
+
+def _split_plan(dev_index, b, h, h_k, max_seqlen, max_res, new_tokens, bits, gs, num_splits):
+    """(split count, workspace bytes) of a decode call on the current device; both are pure functions of
+    these arguments (and of the device's compute-unit count), so the two library calls are made once."""
+    key = (dev_index, b, h, h_k, max_seqlen, max_res, new_tokens, bits, gs, num_splits)
+    hit = _SPLIT_PLANS.get(key)
+    if hit is None:
+        L = _lib.lib()
+        ns = num_splits or L.bitdecode_num_splits(b, h_k, max_seqlen, max_res, new_tokens, bits, gs)
+        hit = (ns, L.bitdecode_fwd_workspace_bytes(b, h, ns))
+        if len(_SPLIT_PLANS) >= 4096:
+            _SPLIT_PLANS.clear()
+        _SPLIT_PLANS[key] = hit
+    return hit
 
 
 def _i32_dev(x, b, device, name):
@@ -185,7 +223,7 @@ def kvcache_pack_int(k_cache: torch.Tensor, k_pack: torch.Tensor, k_params: torc
     a.quant_mode = mode
     if paged:
         _set_paging(a, opt_block_table, cb)
-    with torch.cuda.device(device):
+    with _on_device(device):
         _lib.check(_lib.lib().bitdecode_qpack(ctypes.byref(a), _stream_ptr(device)))
 
 
@@ -321,13 +359,10 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
     a.bits, a.group_size, a.dtype = num_bits, group_size, dtype
     a.quant_mode = mode
     a.softmax_scale = float(softmax_scale)
-    L = _lib.lib()
-    with torch.cuda.device(device):
-        ns = int(num_splits)
-        if ns == 0:
-            ns = L.bitdecode_num_splits(b, h_k, a.max_seqlen_k, a.max_res_len, 0, num_bits, group_size)
+    with _on_device(device):
+        ns, nbytes = _split_plan(device.index, b, h, h_k, a.max_seqlen_k, a.max_res_len, 0, num_bits, group_size,
+                                 int(num_splits))
         a.num_splits = ns
-        nbytes = L.bitdecode_fwd_workspace_bytes(b, h, ns)
         if nbytes:
             # zero-filled: the arrival counters at its head must be 0 before the first call
             # (every call leaves them at 0 again)
@@ -366,7 +401,7 @@ def fwd_kvcache_int(q: torch.Tensor,
     # (the reference allocates its accumulators per call, decode_api.cpp:292-295, 375-390)
     plan = plan_fwd_kvcache_int(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale,
                                 quant_mode, group_size, num_bits, _stream_ws=True, **kwargs)
-    with torch.cuda.device(plan.device):
+    with _on_device(plan.device):
         plan.run()
     return (plan.out, plan.lse) if return_lse else plan.out
 
@@ -413,7 +448,7 @@ def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: tor
     a.v_new, a.vnew_stride_b, a.vnew_stride_h = v_new.data_ptr(), v_new.stride(0), v_new.stride(2)
     a.max_len = max_len
     L = _lib.lib()
-    with torch.cuda.device(device):
+    with _on_device(device):
         ns = int(num_splits)
         if ns == 0:
             ns = L.bitdecode_num_splits(b, h_k, max_len // CHUNK * CHUNK, CHUNK, 0, num_bits, group_size)
@@ -452,6 +487,6 @@ def fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Te
     plan = plan_fwd_kvcache_int_append(q, k_new, v_new, k_pack, k_params, v_pack, v_params, k_residual, v_residual,
                                        lengths, max_len, opt_block_table, softmax_scale, quant_mode, group_size,
                                        num_bits, _stream_ws=True, **kwargs)
-    with torch.cuda.device(plan.device):
+    with _on_device(plan.device):
         plan.run()
     return (plan.out, plan.lse) if return_lse else plan.out
