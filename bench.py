@@ -86,14 +86,36 @@ def alloc_cache(b, S, h_k, bits, gs, dev):
             torch.zeros((b, 128 // gs, h_k, S), dtype=torch.float32, device=dev))
 
 
-def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, replays=1):
-    """Returns (wall seconds, event seconds, graphed) for `steps` steps, the captured graph of `steps`
-    steps being replayed `replays` times inside the timed region (both times are totals over
-    steps * replays steps; without a graph the eager loop runs steps * replays steps)."""
+MIN_GRAPH_NODES = 200      # steps captured into one graph (a multiple of --steps): keeps the gaps between graph launches rare
+MIN_TIMED_STEPS = 400      # steps inside the timed region
+WARM_STEPS = 1600          # untimed replayed steps in front of it: the first ~10 ms after idle run 3-10 % slower
+
+
+def slots_needed(steps, warmup, limit):
+    """Smallest number of slots such that, when time_steps(..., steady=True) hands step i to slot i % slots
+    (eager warm-up, capture, every replay of the graph restarting at i = 0), no slot is used more than
+    `limit` times."""
+    nodes = steps * max(1, math.ceil(MIN_GRAPH_NODES / steps))
+    plays = 1 + math.ceil(WARM_STEPS / nodes) + max(1, math.ceil(MIN_TIMED_STEPS / nodes))
+    n = 1
+    while math.ceil(warmup / n) + 1 + plays * math.ceil(nodes / n) > limit:
+        n += 1
+    return n
+
+
+def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True):
+    """Times `run_step`.  Eager warm-up of `warmup` steps, then one HIP graph of `nodes` steps (`steps` times
+    a whole number, at least MIN_GRAPH_NODES when `steady`) is captured, replayed untimed (once to upload it,
+    then for WARM_STEPS steps when `steady`) and replayed `replays` times between two events and two host
+    synchronisations.  Without a graph the eager loop runs the same number of steps.  Returns a dict with the
+    wall and event time per step and what was run."""
     dev = torch.device("cuda:0")
     for i in range(warmup):
         run_step(i)
     torch.cuda.synchronize(dev)
+    nodes = steps * (max(1, math.ceil(MIN_GRAPH_NODES / steps)) if steady else 1)
+    replays = max(1, math.ceil(MIN_TIMED_STEPS / nodes)) if steady else 1
+    warm = math.ceil(WARM_STEPS / nodes) if steady else 0
     graph = None
     if use_graph:
         try:
@@ -104,13 +126,17 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, replays=1):
             torch.cuda.current_stream(dev).wait_stream(side)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                for i in range(steps):
+                for i in range(nodes):
                     run_step(i)
-            graph.replay()          # untimed: first replay uploads the graph
+            for _ in range(1 + warm):
+                graph.replay()          # untimed: the first replay uploads the graph
             torch.cuda.synchronize(dev)
         except Exception as e:      # noqa: BLE001
             print(f"[bench] graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
             graph = None
+    if graph is None:
+        for i in range(warm * nodes):
+            run_step(i)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize(dev)
     t0 = time.perf_counter()
@@ -119,11 +145,16 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, replays=1):
         for _ in range(replays):
             graph.replay()
     else:
-        for i in range(steps * replays):
+        for i in range(nodes * replays):
             run_step(i)
     e1.record()
     torch.cuda.synchronize(dev)
     t1 = time.perf_counter()
+    timed = nodes * replays
+    res = {"wall_us": (t1 - t0) / timed * 1e6, "event_us": e0.elapsed_time(e1) * 1e3 / timed,
+           "graphed": graph is not None, "timed_steps": timed, "graph_nodes": nodes if graph is not None else 0,
+           "replays": replays if graph is not None else 0,
+           "untimed_replays": 1 + warm if graph is not None else 0, "quantiles": None}
     if quantile_reps and graph is not None:
         # spread of the per-step time over further replays of the same graph (outside the timed region)
         per_step = []
@@ -133,11 +164,11 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, replays=1):
             graph.replay()
             b_.record()
             torch.cuda.synchronize(dev)
-            per_step.append(a.elapsed_time(b_) * 1e3 / steps)
+            per_step.append(a.elapsed_time(b_) * 1e3 / nodes)
         per_step.sort()
         pick = lambda f: round(per_step[min(len(per_step) - 1, int(f * len(per_step)))], 3)
-        time_steps.last_quantiles = {"p20": pick(0.2), "p50": pick(0.5), "p80": pick(0.8), "replays": quantile_reps}
-    return t1 - t0, e0.elapsed_time(e1) * 1e-3, graph is not None
+        res["quantiles"] = {"p20": pick(0.2), "p50": pick(0.5), "p80": pick(0.8), "replays": quantile_reps}
+    return res
 
 
 def cpu_baseline(q, k, v, S, R, bits, gs, scale, budget_s=20.0):
@@ -247,12 +278,11 @@ def main():
         torch.cuda.synchronize(dev)
         del src, dst
 
-    # A short run (the default driver call is --steps 20) replays its graph often enough that the one host
-    # synchronisation at the end of the timed region is spread over at least 400 steps
-    replays = max(1, math.ceil(400 / args.steps))
-    wall, evs, graphed = time_steps(step, args.steps, args.warmup, not args.no_graph, quantile_reps=15, replays=replays)
-    us_step = wall / (args.steps * replays) * 1e6
-    us_step_ev = evs / (args.steps * replays) * 1e6
+    # Whatever --steps is, the timed region holds at least MIN_TIMED_STEPS steps in graphs of at least
+    # MIN_GRAPH_NODES steps, so the host synchronisation at its end and the gaps between graph launches
+    # stay below 1 % of it; `steps` in the JSON line is the command line's value, `config` says what ran.
+    T = time_steps(step, args.steps, args.warmup, not args.no_graph, quantile_reps=15)
+    us_step, us_step_ev, graphed = T["wall_us"], T["event_us"], T["graphed"]
     achieved = total_bytes / (us_step_ev * 1e-6) / 1e9
 
     result = {
@@ -275,16 +305,17 @@ def main():
                    "residual_tokens": win_len.tolist() if ragged else R, "bits": bits, "group_size": gs,
                    "num_splits": plans[0].num_splits, "kv_buffers_rotated": nbuf,
                    "launch": "hip-graph" if graphed else "eager",
-                   "timed_steps": args.steps * replays,
-                   "graph_replays_in_timed_region": replays if graphed else 0},
+                   "timed_steps": T["timed_steps"], "steps_per_graph": T["graph_nodes"],
+                   "graph_replays_in_timed_region": T["replays"],
+                   "untimed_graph_replays_before": T["untimed_replays"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.num_splits == 0 else None,
                      "kernel": "fwd_splitkv_kernel", "algorithmic_bytes": total_bytes,
                      "packed_stream_bytes": packed_bytes, "us_per_step_events": round(us_step_ev, 3)},
     }
-    if getattr(time_steps, "last_quantiles", None):
-        result["us_per_step_quantiles"] = time_steps.last_quantiles
+    if T["quantiles"]:
+        result["us_per_step_quantiles"] = T["quantiles"]
 
     if not args.no_probe:
         # what the memory system alone allows: a kernel that only reads as many bytes as one step streams
@@ -299,8 +330,7 @@ def main():
             buf = probe_bufs[i % nbuf]
             _lib.check(L.bitdecode_read_probe(buf.data_ptr(), probe_bytes, None, torch.cuda.current_stream(dev).cuda_stream))
 
-        _, epr, _ = time_steps(probe, args.steps, args.warmup, not args.no_graph, replays=replays)
-        us_probe = epr / (args.steps * replays) * 1e6
+        us_probe = time_steps(probe, args.steps, args.warmup, not args.no_graph)["event_us"]
         result["roofline"]["read_kernel_us"] = round(us_probe, 3)
         result["roofline"]["read_kernel_GBs"] = round(probe_bytes / (us_probe * 1e-6) / 1e9, 1)
         result["roofline"]["frac_of_read_kernel"] = round(us_probe / us_step_ev, 4)
@@ -319,8 +349,7 @@ def main():
                             num_splits=args.num_splits, out=outs[j])
 
         n_drop = max(50, args.steps)
-        w_d, e_d, _ = time_steps(dropin, n_drop, 5, False)
-        result["dropin_eager_us_per_call"] = round(e_d / n_drop * 1e6, 3)
+        result["dropin_eager_us_per_call"] = round(time_steps(dropin, n_drop, 5, False, steady=False)["event_us"], 3)
         result["dropin_eager_note"] = ("fwd_kvcache_int(...) called %d times in a Python loop, GPU time between first "
                                        "and last call / calls; bound by the host's per-call work (argument checks, "
                                        "ctypes), not by the kernel" % n_drop)
@@ -348,9 +377,8 @@ def main():
                                  "k-channel", gs, bits, dst_offset=S - 128)
 
         n_pack = max(10, args.steps // 4)
-        _, ep, _ = time_steps(pack_all, n_pack, 3, not args.no_graph)
-        _, ea, _ = time_steps(pack_block, args.steps, args.warmup, not args.no_graph)
-        us_pack, us_app = ep / n_pack * 1e6, ea / args.steps * 1e6
+        us_pack = time_steps(pack_all, n_pack, 3, not args.no_graph)["event_us"]
+        us_app = time_steps(pack_block, args.steps, args.warmup, not args.no_graph)["event_us"]
         rd = b * h_k * S * 128 * 2 * 2
         wr = int(b * h_k * S * 128 * 2 * (bits / 8 + 4 / gs))      # the whole capacity is packed
         gbs = (rd + wr) / (us_pack * 1e-6) / 1e9
@@ -364,9 +392,9 @@ def main():
     if not args.no_step:
         # the same decode as one launch that also appends the step's new token (device-side lengths).  A slot
         # is a packed cache with a window and a length counter of its own, starting at S packed tokens + 64 in
-        # the window; there are enough slots that none sees 60 steps (warm-up, the untimed first replay and
-        # the timed replay together), so no window fills inside the measurement
-        n_slots = max(nbuf, math.ceil((2 * args.steps + args.warmup) / 59))
+        # the window; there are enough slots that none sees 60 steps (warm-up, capture, untimed and timed
+        # replays together), so no window fills inside the measurement
+        n_slots = max(nbuf, slots_needed(args.steps, args.warmup, 59))
         splans = []
         for i in range(n_slots):
             cache, kres, vres = keep[i % nbuf]
@@ -376,9 +404,9 @@ def main():
             splans.append(plan_fwd_kvcache_int_append(q_t, kn, kn.clone(), *cache, kres.clone(), vres.clone(), lengths,
                                                       S + 127, None, scale, "k-channel", gs, bits,
                                                       num_splits=args.num_splits))
-        _, est, _ = time_steps(lambda i: splans[i % n_slots].run(), args.steps, args.warmup, not args.no_graph)
+        us_append = time_steps(lambda i: splans[i % n_slots].run(), args.steps, args.warmup, not args.no_graph)["event_us"]
         result["decode_step_with_append"] = {
-            "entry": "bitdecode_fwd_append", "us_per_step": round(est / args.steps * 1e6, 3),
+            "entry": "bitdecode_fwd_append", "us_per_step": round(us_append, 3),
             "window_tokens": "65-123", "does": "attend + store the new token + advance the device-side length"}
         del splans
 
@@ -395,8 +423,7 @@ def main():
             fplans.append((plan_fwd_kvcache_int(q.to(dev), *dummy, None, scale, "k-channel", gs, bits, seqlen_k=0,
                                                 k_residual=kd, v_residual=vd, **kw16), q.to(dev), kd, vd))
         torch.cuda.synchronize(dev)
-        w16, e16, _ = time_steps(lambda i: fplans[i % nb16][0].run(), args.steps, args.warmup, not args.no_graph)
-        us16 = e16 / args.steps * 1e6
+        us16 = time_steps(lambda i: fplans[i % nb16][0].run(), args.steps, args.warmup, not args.no_graph)["event_us"]
         fp16_tokens = int((packed_len + win_len).sum()) if ragged else b * (S + R)
         fp16_bytes = fp16_tokens * h_k * 128 * 2 * 2 + 2 * b * h * 128 * 2
 
@@ -407,8 +434,7 @@ def main():
         try:
             if ragged:
                 raise RuntimeError("not run on a ragged batch (SDPA would attend the padding as well)")
-            _, es, _ = time_steps(sdpa, max(10, args.steps // 4), 3, False)
-            us_sdpa = es / max(10, args.steps // 4) * 1e6
+            us_sdpa = time_steps(sdpa, max(10, args.steps // 4), 3, False, steady=False)["event_us"]
         except Exception as e:  # noqa: BLE001
             print(f"[bench] torch SDPA baseline failed: {e}", file=sys.stderr)
             us_sdpa = None
