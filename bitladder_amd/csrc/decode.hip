@@ -8,9 +8,9 @@
 //    16-token tiles of the fp16 window.  A unit is fetched with ten direct-to-LDS loads
 //    (global_load_lds_dwordx4: 64 lanes x 16 B = one contiguous 1 KB row each, no staging
 //    registers) into the wave's private LDS region and read back 16 bytes per lane just before
-//    it is unpacked; the next unit of the wave is requested from inside the current one, as soon
-//    as the rows it will overwrite have been read.  With no load-staging registers the kernel
-//    fits 3-4 waves per SIMD: a wave that waits for its unit leaves the VALU to the others.
+//    it is unpacked.  The rows are requested in the order they are consumed, a few ahead of the
+//    one being read and running on into the wave's next unit.  With no load-staging registers the
+//    kernel fits 3-4 waves per SIMD: a wave that waits for a row leaves the VALU to the others.
 //  * Both products are computed transposed on v_mfma_f32_16x16x32_f16:
 //        S^T = K * Q^T   (A = K codes, row = token; B = Q, column = query head of the GQA group)
 //        O^T = V^T * P^T (A = V codes, row = channel; B = P^T)
@@ -33,9 +33,9 @@
 //  * Online softmax in base 2 per head (softmax.h:250-310) in steps of 64 tokens: running max
 //    shared by the four lanes of a head through two lane-half swaps, accumulators rescaled only
 //    when some head's max actually moved.
-//  * The waves of a workgroup merge through LDS; splits merge in the same launch: every
-//    workgroup publishes its unnormalised (O, max, sum) and the one that draws the last ticket
-//    of a (batch, kv-head) combines all of them.
+//  * The waves of a workgroup merge through LDS, one wave per query head; splits merge in the
+//    same launch: that wave publishes the head's unnormalised (O, max, sum), draws a ticket from
+//    the head's counter, and the wave that draws the last one combines all splits of the head.
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -44,6 +44,7 @@
 #include "layout.h"
 #include "qpack_chunk.h"
 
+// rows a wave keeps in flight (see "the rows of a unit as a pipeline")
 #ifndef X_DEPTH
 #define X_DEPTH 4
 #endif
@@ -435,13 +436,9 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
         (const __attribute__((address_space(3))) void*)p));
 }
 
-// The loads of a unit, in the order they are consumed: K side (K parameters, four K code rows), then
-// V side (V parameters, four V code rows).  A wave issues both sides of its first unit at once.
-// After that the next unit's K side is issued as soon as the current unit's last QK^T has read the
-// K rows (and the data of those reads has come back: wait_lds_reads), into the same rows and into
-// the other K-parameter slot, and its V side as soon as the last PV has read the V rows and V
-// parameters: the next unit is on its way while the current one is being computed, without a
-// second code buffer.
+// Base addresses of one unit of one (batch, kv-head): K codes, V codes, K parameters, V parameters.  The
+// rows behind them are fetched one by one in the order they are consumed (see "the rows of a unit as a
+// pipeline" below).
 template <int BITS, int GS>
 struct UnitAddr {
     const uint8_t* kc;
