@@ -1134,7 +1134,11 @@ __device__ __forceinline__ bool step_overflows(int capacity, int t) {
 // The workgroup that writes the output of a (batch, kv-head) is the last one of that pair to use the
 // length and the window.  One of its threads draws a ticket as soon as that is settled; the holder of
 // the last of the h_k tickets of a sequence knows that every workgroup of the sequence has read the
-// length, advances it and resets the counter.
+// length, advances it and resets the counter.  The tickets are relaxed device-scope atomics performed at the
+// memory side (totally ordered); no data written in this launch is read through them, so no release or
+// acquire is involved.  The new length and the reset counter are read again only by the next launch on the
+// stream, and the end of a kernel makes plain stores visible to it: both may be plain stores, provided lengths
+// and counters live in ordinary device memory (not host-coherent or fine-grained memory polled by another agent).
 __device__ __forceinline__ void step_ticket(int* step_tickets, int* lengths, int n_heads_k, int capacity, int bi, int t) {
     const int drawn = __hip_atomic_fetch_add(&step_tickets[bi * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (drawn == n_heads_k - 1) {
