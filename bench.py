@@ -262,8 +262,10 @@ def main():
                                         k_residual=kres, v_residual=vres, num_splits=args.num_splits)
         plans.append(plan)
         keep.append((cache, kres, vres))
-        if i < 2 and not args.no_qpack:
-            srcs.append((kd, vd))      # fp16 sources of the first two caches, for the quantize-pack leg
+        if not args.no_qpack and (i < 2 or sum(a.numel() + b_.numel() for a, b_ in srcs) * 2 < 640e6):
+            # fp16 sources for the quantize-pack leg: at least two, and enough of them (more than twice the
+            # 256 MB Infinity Cache in total) that no pack call finds its input cached
+            srcs.append((kd, vd))
         del kd, vd
     torch.cuda.synchronize(dev)
 

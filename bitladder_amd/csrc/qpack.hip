@@ -12,7 +12,7 @@
 namespace bitdecode {
 namespace {
 
-template <int BITS, int GS, bool BF16, bool KT>
+template <int BITS, int GS, bool BF16, bool KT, bool STREAM>
 __global__ __launch_bounds__(qp::kPackThreads) void qpack_kernel(QpackParams P) {
     __shared__ qp::PackLds<GS> L;
     const int tid = threadIdx.x;
@@ -31,31 +31,36 @@ __global__ __launch_bounds__(qp::kPackThreads) void qpack_kernel(QpackParams P) 
     // 4 bits, group 128: with the V tile prefetched the kernel needs 133 registers and only three
     // workgroups fit a CU; fetched after the K side it needs 114, a fourth workgroup fits (LDS: 40 KB
     // each) and the kernel is 10 % faster.  (At group 64 a fourth workgroup was measured 3 % slower.)
-    qp::pack_chunk<BITS, GS, BF16, !(BITS == 4 && GS == 128), KT>(
+    qp::pack_chunk<BITS, GS, BF16, !(BITS == 4 && GS == 128), KT, STREAM>(
         L, tid, true, [=](int n) { return ks + n * k_st; }, [=](int n) { return vs + n * v_st; }, D);
+}
+
+template <int BITS, int GS, bool KT, bool STREAM>
+hipError_t launch_qpack_tt(const QpackParams& P, dim3 grid, hipStream_t stream) {
+    if (P.bf16) {
+        hipLaunchKernelGGL((qpack_kernel<BITS, GS, true, KT, STREAM>), grid, dim3(256), 0, stream, P);
+    } else {
+        hipLaunchKernelGGL((qpack_kernel<BITS, GS, false, KT, STREAM>), grid, dim3(256), 0, stream, P);
+    }
+    return hipGetLastError();
 }
 
 template <int BITS, int GS>
 hipError_t launch_qpack_t(const QpackParams& P, hipStream_t stream) {
     dim3 grid(P.n_tokens / kChunk, P.hk, P.b);
+    // a bulk pack (more chunks than two rounds of workgroups over the 256 compute units) streams its input
+    // and output past the caches; an append of a block per sequence does not
+    const bool stream_data = static_cast<int64_t>(grid.x) * grid.y * grid.z >= 512;
     if (P.ktensor) {      // K quantized per token like V: 4 bits only, as in the reference (qpack.h:385)
         if constexpr (BITS == 4) {
-            if (P.bf16) {
-                hipLaunchKernelGGL((qpack_kernel<BITS, GS, true, true>), grid, dim3(256), 0, stream, P);
-            } else {
-                hipLaunchKernelGGL((qpack_kernel<BITS, GS, false, true>), grid, dim3(256), 0, stream, P);
-            }
-            return hipGetLastError();
+            return stream_data ? launch_qpack_tt<BITS, GS, true, true>(P, grid, stream)
+                               : launch_qpack_tt<BITS, GS, true, false>(P, grid, stream);
         } else {
             return hipErrorInvalidValue;
         }
     }
-    if (P.bf16) {
-        hipLaunchKernelGGL((qpack_kernel<BITS, GS, true, false>), grid, dim3(256), 0, stream, P);
-    } else {
-        hipLaunchKernelGGL((qpack_kernel<BITS, GS, false, false>), grid, dim3(256), 0, stream, P);
-    }
-    return hipGetLastError();
+    return stream_data ? launch_qpack_tt<BITS, GS, false, true>(P, grid, stream)
+                       : launch_qpack_tt<BITS, GS, false, false>(P, grid, stream);
 }
 
 }  // namespace

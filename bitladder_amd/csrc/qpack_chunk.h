@@ -152,10 +152,25 @@ __device__ __forceinline__ void row_group_stats(const uint16_t* tile, int tid, S
     }
 }
 
+// 16-byte global load / store of the chunk routine.  STREAM marks data that is touched once (the bulk pack of
+// a long prefix: fp16 rows in, packed rows out) with the non-temporal hint: 11-13 % faster there.  A pack of a
+// single block per sequence keeps the default policy: its output is read by the very next decode step, and the
+// small launch ends sooner when its stores may complete in the cache (6.5 against 7.4-8.0 us).
+template <bool STREAM>
+__device__ __forceinline__ u4 ld16(const void* p) {
+    if constexpr (STREAM) return __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+    else return *reinterpret_cast<const u4*>(p);
+}
+template <bool STREAM>
+__device__ __forceinline__ void st16(void* p, u4 v) {
+    if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u4*>(p));
+    else *reinterpret_cast<u4*>(p) = v;
+}
+
 // With KT ("k-tensor" mode, qpack.h:378-470 of the reference) K is quantized like V, per token over groups
 // of GS channels; its codes keep the K layout, its parameters go per chunk as
 // [64-token half][channel group][16-token tile][token] (scale, zero) pairs.
-template <int BITS, int GS, bool BF16, bool PREFETCH_V, bool KT = false, class RowK, class RowV>
+template <int BITS, int GS, bool BF16, bool PREFETCH_V, bool KT = false, bool STREAM = false, class RowK, class RowV>
 __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active, RowK krow, RowV vrow,
                                            const ChunkDst& D) {
 #pragma clang fp contract(off)
@@ -168,10 +183,10 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
     u4 kreg[8], vreg[8];
     if (active) {
 #pragma unroll
-        for (int x = 0; x < 8; ++x) kreg[x] = *reinterpret_cast<const u4*>(krow(lrow + 16 * x) + lcol);
+        for (int x = 0; x < 8; ++x) kreg[x] = ld16<STREAM>(krow(lrow + 16 * x) + lcol);
 #pragma unroll
         for (int x = 0; x < 8; ++x) {
-            if constexpr (PREFETCH_V) vreg[x] = *reinterpret_cast<const u4*>(vrow(lrow + 16 * x) + lcol);
+            if constexpr (PREFETCH_V) vreg[x] = ld16<STREAM>(vrow(lrow + 16 * x) + lcol);
         }
 #pragma unroll
         for (int x = 0; x < 8; ++x) *reinterpret_cast<u4*>(&tile[(lrow + 16 * x) * kRowHalves + lcol]) = kreg[x];
@@ -255,7 +270,7 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
                     }
                     out[j] = w;
                 }
-                *reinterpret_cast<u4*>(kc + t * 1024 + l * 16) = out;
+                st16<STREAM>(kc + t * 1024 + l * 16, out);
             }
         } else {
             const int tp = tid >> 6, l = tid & 63, m = l & 15, kg = l >> 4;
@@ -279,7 +294,7 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
                     out[2 * tin + jj] = w;
                 }
             }
-            *reinterpret_cast<u4*>(kc + tp * 1024 + l * 16) = out;
+            st16<STREAM>(kc + tp * 1024 + l * 16, out);
         }
     }
     __syncthreads();
@@ -288,7 +303,7 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
     if (active) {
 #pragma unroll
         for (int x = 0; x < 8; ++x) {
-            if constexpr (!PREFETCH_V) vreg[x] = *reinterpret_cast<const u4*>(vrow(lrow + 16 * x) + lcol);
+            if constexpr (!PREFETCH_V) vreg[x] = ld16<STREAM>(vrow(lrow + 16 * x) + lcol);
         }
 #pragma unroll
         for (int x = 0; x < 8; ++x) *reinterpret_cast<u4*>(&tile[(lrow + 16 * x) * kRowHalves + lcol]) = vreg[x];
@@ -329,7 +344,7 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
                     }
                     out[x] = w;
                 }
-                *reinterpret_cast<u4*>(vc + sb * 2048 + hf * 1024 + l * 16) = out;
+                st16<STREAM>(vc + sb * 2048 + hf * 1024 + l * 16, out);
             }
         } else {
             const int sb2 = tid >> 7, hf = (tid >> 6) & 1, l = tid & 63, c = l & 15, kg = l >> 4;
@@ -349,7 +364,7 @@ __device__ __forceinline__ void pack_chunk(PackLds<GS>& L, int tid, bool active,
                 }
                 out[x] = w;
             }
-            *reinterpret_cast<u4*>(vc + sb2 * 2048 + hf * 1024 + l * 16) = out;
+            st16<STREAM>(vc + sb2 * 2048 + hf * 1024 + l * 16, out);
         }
     }
 }
