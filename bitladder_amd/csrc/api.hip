@@ -254,6 +254,14 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
     if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim * sizeof(float) >= (size_t(1) << 31))
         return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d heads: partial outputs of 2 GiB or more", nsplit, a->b, a->h);
+    // the kernel divides workgroup ids and unit counts by the split count and the head count with a
+    // multiply (kernels.h: division_magic), exact while numerator x divisor stays below 2^32
+    {
+        const uint64_t wgs = static_cast<uint64_t>(nsplit) * a->b * a->h_k;
+        const uint64_t units = static_cast<uint64_t>(max_s) / 64 + static_cast<uint64_t>(nsplit);
+        if (wgs * std::max(nsplit, a->h_k) >= (1ull << 32) || units * nsplit >= (1ull << 32))
+            return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d kv heads: too many workgroups", nsplit, a->b, a->h_k);
+    }
     if (static_scratch) {
         const size_t rows = static_cast<size_t>(a->b) * a->h;
         const size_t need = nsplit > 1 ? static_cast<size_t>(nsplit) * rows * (kHeadDim + 2) * sizeof(float) : 0;
@@ -297,6 +305,8 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     P.scale_log2 = fabsf(a->softmax_scale) * 1.4426950408889634f;   // decode_api.cpp:128-142
     P.neg_scale = a->softmax_scale < 0.0f;
     P.xcd_remap = (a->b * a->h_k) % 8 == 0 && nsplit > 1;
+    P.nsplit_magic = division_magic(static_cast<uint32_t>(nsplit));
+    P.hk_magic = division_magic(static_cast<uint32_t>(a->h_k));
     P.block_table = a->block_table; P.bt_stride = a->block_table_stride;
     P.chunks_per_page = a->block_table ? a->cache_tokens / kChunk : 1;
     P.bits = a->bits; P.gs = a->group_size; P.bf16 = a->dtype == BITDECODE_BF16;

@@ -109,6 +109,11 @@ __device__ __forceinline__ h8 cvt_h8(u4 raw) {
     }
 }
 
+// n / d with the host's magic number for d (kernels.h)
+__device__ __forceinline__ int div_magic(int n, uint32_t magic) {
+    return magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(n), magic)) : n;
+}
+
 __device__ __forceinline__ u4 ld_u4(const void* p) { return *reinterpret_cast<const u4*>(p); }
 // the same with the non-temporal hint, for rows that are read once and whole by one instruction
 __device__ __forceinline__ u4 ld_u4_stream(const void* p) { return __builtin_nontemporal_load(reinterpret_cast<const u4*>(p)); }
@@ -1251,14 +1256,15 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         int bhid;
         if (P.xcd_remap) {
             const int xcd = lin & 7, r = lin >> 3;
-            bhid = (r / P.nsplit) * 8 + xcd;
-            split = r % P.nsplit;
+            const int q = div_magic(r, P.nsplit_magic);
+            bhid = q * 8 + xcd;
+            split = r - q * P.nsplit;
         } else {
-            bhid = lin / P.nsplit;
-            split = lin % P.nsplit;
+            bhid = div_magic(lin, P.nsplit_magic);
+            split = lin - bhid * P.nsplit;
         }
-        bi = bhid / P.hk;
-        hk = bhid % P.hk;
+        bi = div_magic(bhid, P.hk_magic);
+        hk = bhid - bi * P.hk;
     }
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: unit addresses stay in SGPRs
@@ -1280,7 +1286,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         R = P.reslens ? min(max(P.reslens[bi], 0), P.res_cap) : P.reslen;
     }
     const int nU = (S / kChunk) * C::UPC;
-    const int ups = (nU + P.nsplit - 1) / P.nsplit;
+    const int ups = div_magic(nU + P.nsplit - 1, P.nsplit_magic);
     const int u0 = min(nU, split * ups);
     const int u1 = min(nU, u0 + ups);
     const int nT = (R + 15) / 16;

@@ -72,7 +72,12 @@ struct FwdParams {
     int64_t knew_sb, knew_sh, vnew_sb, vnew_sh;
     int capacity;               // packed tokens a sequence can hold (set for every call; clamps device-side lengths)
     int res_cap;                // rows of the fp16 window (clamps device-side window lengths)
+    // n / nsplit and n / hk as one multiply: magic = ceil(2^32 / d), or 0 for d = 1; exact for n * d < 2^32
+    // (a runtime integer division costs the prologue of every workgroup some 100 cycles, and there were five)
+    uint32_t nsplit_magic, hk_magic;
 };
+
+inline uint32_t division_magic(uint32_t d) { return d <= 1 ? 0u : static_cast<uint32_t>(((1ull << 32) + d - 1) / d); }
 
 hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);
 hipError_t launch_fwd(const FwdParams& p, hipStream_t stream);
