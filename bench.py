@@ -41,6 +41,15 @@ WORKLOADS = {
     "llama2-7b-mha-4k-4bit-g128": (1, 32, 32, 4096, 128, 4, 128, torch.float16),
     "llama3-8b-gqa-128k-2bit-g64": (1, 32, 8, 131072, 128, 2, 64, torch.float16),
     "llama3-70b-gqa-64k-2bit-g128-b8": (8, 64, 8, 65536, 128, 2, 128, torch.bfloat16),
+    # further shapes, used to tune the launch heuristics (not BASELINE configurations)
+    "llama3-8b-gqa-128k-4bit-g128": (1, 32, 8, 131072, 128, 4, 128, torch.float16),
+    "llama3-8b-gqa-8k-4bit-g128-b16": (16, 32, 8, 8192, 128, 4, 128, torch.float16),
+    "llama3-70b-gqa-64k-4bit-g128-b8": (8, 64, 8, 65536, 128, 4, 128, torch.bfloat16),
+    "llama3-8b-gqa-96k-4bit-g128": (1, 32, 8, 98304, 128, 4, 128, torch.float16),
+    "llama3-8b-gqa-64k-4bit-g128": (1, 32, 8, 65536, 128, 4, 128, torch.float16),
+    "llama3-8b-gqa-48k-4bit-g128": (1, 32, 8, 49152, 128, 4, 128, torch.float16),
+    "llama3-8b-gqa-16k-4bit-g128-b4": (4, 32, 8, 16384, 128, 4, 128, torch.float16),
+    "llama3-8b-gqa-8k-4bit-g128-b4": (4, 32, 8, 8192, 128, 4, 128, torch.float16),
     # ragged batch: 16 sequences of seeded lengths in [1024, 8192]; S is the cache capacity, R the window
     # capacity.  Whole 128-token blocks of a sequence are packed; the remainder (< 128) plus the 128 newest
     # tokens stay in the fp16 window (128-255 tokens), as in a decode loop just before the next block is packed.

@@ -317,7 +317,8 @@ __device__ __forceinline__ void step_probabilities_shared(const f4 (&sc)[4], uin
 // ---------------------------------------------------------------------------------------------
 // packed units, streamed through LDS
 // ---------------------------------------------------------------------------------------------
-template <int BITS, int GS>
+// FEW: the variant with 8 waves per workgroup and a deeper row pipeline (see launch_fwd_tt)
+template <int BITS, int GS, bool FEW = false>
 struct UnitCfg {
     static constexpr int UT = unit_tokens(BITS);             // tokens per unit (4 KB of K codes, 4 KB of V codes)
     static constexpr int UPC = kChunk / UT;                  // units per 128-token chunk
@@ -338,8 +339,9 @@ struct UnitCfg {
     // LDS region of a wave: K rows | V rows | K parameters, two slots | V parameters
     static constexpr int OFF_KP = 8192, OFF_VP = 8192 + 2 * KPB;
     static constexpr int REGION = unit_region_bytes(BITS, GS);
-    static constexpr int NW = decode_waves(BITS, GS);        // waves per workgroup
-    static constexpr int DEPTH = (X_DEPTH) < NKP + RPS + 1 ? (X_DEPTH) : NKP + RPS + 1;   // rows a wave keeps in flight
+    static constexpr int NW = FEW ? 8 : decode_waves(BITS, GS);        // waves per workgroup
+    static constexpr int WANT_DEPTH = FEW ? 6 : (X_DEPTH);
+    static constexpr int DEPTH = WANT_DEPTH < NKP + RPS + 1 ? WANT_DEPTH : NKP + RPS + 1;   // rows a wave keeps in flight
     static_assert(REGION == OFF_VP + VPB && REGION % 256 == 0, "region layout");
     static_assert(KPB_T <= KPB && (KPB_T + 1023) / 1024 == NKP, "the per-token K parameters use the same rows");
     static_assert(NW % 4 == 0, "the merge reads four wave weights per LDS access");
@@ -571,21 +573,21 @@ __device__ __forceinline__ void issue_row(const UnitAddr<BITS, GS>& A, uint32_t 
     }
 }
 // prologue of a wave: rows 0 .. kDepth-2 of its first unit
-template <int BITS, int GS, bool KT = false, int I = 0>
+template <int BITS, int GS, bool KT = false, bool FEW = false, int I = 0>
 __device__ __forceinline__ void issue_first_rows(const UnitAddr<BITS, GS>& A, uint32_t lane16, uint32_t region) {
-    if constexpr (I < UnitCfg<BITS, GS>::DEPTH - 1) {
+    if constexpr (I < UnitCfg<BITS, GS, FEW>::DEPTH - 1) {
         issue_row<BITS, GS, I, KT>(A, lane16, region, 0);
-        issue_first_rows<BITS, GS, KT, I + 1>(A, lane16, region);
+        issue_first_rows<BITS, GS, KT, FEW, I + 1>(A, lane16, region);
     }
 }
 // In front of the read of row I of the current unit: send the row that keeps the pipeline full (of this
 // unit, or of the next one if there is one), then wait until row I has landed.  The load may overwrite
 // rows read earlier: every LDS read issued so far has to have returned its data first (a read that has
 // only been issued can be overtaken by the load's write).
-template <int BITS, int GS, bool HAS_NEXT, int I, bool KT = false>
+template <int BITS, int GS, bool HAS_NEXT, int I, bool KT = false, bool FEW = false>
 __device__ __forceinline__ void row_ready(const UnitAddr<BITS, GS>& cur, const UnitAddr<BITS, GS>& next, uint32_t lane16,
                                           uint32_t region, int kslot) {
-    using C = UnitCfg<BITS, GS>;
+    using C = UnitCfg<BITS, GS, FEW>;
     constexpr int ROWS = C::KSIDE + C::VSIDE, kDepth = C::DEPTH, J = I + kDepth - 1;
     // rows of the next unit fetched from inside this one land on K-side rows only: the V parameters of this
     // unit are still in use up to its last row
@@ -690,7 +692,7 @@ __device__ __forceinline__ TokenQ<NCG> token_q(const QRows& Q) {
     return T;
 }
 
-template <int BITS, int GS, bool BF16, bool HAS_NEXT, bool KT = false>
+template <int BITS, int GS, bool BF16, bool HAS_NEXT, bool KT = false, bool FEW = false>
 __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region_lds, int kslot,
                                              const UnitAddr<BITS, GS>& cur, const UnitAddr<BITS, GS>& next,
                                              const QRows& Q, const FwdParams& P, int lane, bool lo_part, const Magic& mg,
@@ -707,7 +709,7 @@ __device__ __forceinline__ void compute_unit(const uint8_t* reg, uint32_t region
     const u4* vcode = reinterpret_cast<const u4*>(reg + 4096) + lane;
     const uint8_t* kpar = reg + C::OFF_KP + kslot * C::KPB;
     const uint8_t* vpar = reg + C::OFF_VP + kg * 16;
-#define ROW_READY(kind, idx) row_ready<BITS, GS, HAS_NEXT, pos_of<BITS, GS>(kind, idx), KT>(cur, next, lane16, region_lds, kslot)
+#define ROW_READY(kind, idx) row_ready<BITS, GS, HAS_NEXT, pos_of<BITS, GS>(kind, idx), KT, FEW>(cur, next, lane16, region_lds, kslot)
 
     // the K parameters lead the queue: the first K group is prepared while the code rows arrive
 #pragma unroll
@@ -1227,16 +1229,16 @@ __device__ __forceinline__ void step_end(uint8_t* lds, int bi, int hk, int t) {
 // [sM, sL: per-wave max and sum, 8 heads x NW floats each][append flag].  A wave's region is reused as its
 // V-transpose slab for fp16 tiles and as its slot of the cross-wave merge buffer (g x 128 floats <= 4 KB).
 // ---------------------------------------------------------------------------------------------
-template <int BITS, int GS>
+template <int BITS, int GS, bool FEW>
 constexpr int fwd_lds_bytes() {
-    using C = UnitCfg<BITS, GS>;
+    using C = UnitCfg<BITS, GS, FEW>;
     return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16;
 }
 
-template <int BITS, int GS, bool BF16, bool APPEND, bool KT>
-__global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
+template <int BITS, int GS, bool BF16, bool APPEND, bool KT, bool FEW>
+__global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
     static_assert(!KT || (BITS == 4 && !APPEND), "per-token K parameters: 4 bits, plain decode");
-    using C = UnitCfg<BITS, GS>;
+    using C = UnitCfg<BITS, GS, FEW>;
     constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     static_assert(sizeof(qp::PackLds<GS>) <= NW * REGION, "the pack tile reuses the wave regions");
@@ -1309,7 +1311,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     UnitAddr<BITS, GS> A;
     if (u < u1) {
         A = unit_addr<BITS, GS, KT>(P, bi, hk, u);
-        issue_first_rows<BITS, GS, KT>(A, lane * 16, region_lds);
+        issue_first_rows<BITS, GS, KT, FEW>(A, lane * 16, region_lds);
         wait_then_take<C::DEPTH - 1>(qa, qb, qa_raw, qb_raw);
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
@@ -1355,11 +1357,11 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
         int kslot = 0;
         for (int un = u + NW; un < u1; un += NW) {        // units that have a successor: it is fetched from inside
             const UnitAddr<BITS, GS> An = unit_addr<BITS, GS, KT>(P, bi, hk, un);
-            compute_unit<BITS, GS, BF16, true, KT>(region, region_lds, kslot, A, An, Q, P, lane, lo_part, mg, st, KQp);
+            compute_unit<BITS, GS, BF16, true, KT, FEW>(region, region_lds, kslot, A, An, Q, P, lane, lo_part, mg, st, KQp);
             A = An;
             kslot ^= 1;
         }
-        compute_unit<BITS, GS, BF16, false, KT>(region, region_lds, kslot, A, A, Q, P, lane, lo_part, mg, st, KQp);
+        compute_unit<BITS, GS, BF16, false, KT, FEW>(region, region_lds, kslot, A, A, Q, P, lane, lo_part, mg, st, KQp);
     }
     PROF(3);
     // ---- fp16 window tiles of this wave (the region becomes the V-transpose slab)
@@ -1511,23 +1513,37 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS>::NW * 64)) void fwd_splitkv_kern
     PROF_FLUSH();
 }
 
-template <int BITS, int GS, bool BF16, bool APPEND, bool KT = false>
-hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
-    constexpr int kLds = fwd_lds_bytes<BITS, GS>();
+template <int BITS, int GS, bool BF16, bool APPEND, bool KT, bool FEW>
+hipError_t launch_fwd_ttt(const FwdParams& P, hipStream_t stream) {
+    constexpr int kLds = fwd_lds_bytes<BITS, GS, FEW>();
     // the dynamic-LDS limit is raised once per kernel and device (idempotent, so a race between
     // two host threads only repeats the call)
     static bool configured[64] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !configured[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT, FEW>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return e;
         if (dev >= 0 && dev < 64) configured[dev] = true;
     }
-    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT>), dim3(P.nsplit * P.hk * P.b),
-                       dim3(UnitCfg<BITS, GS>::NW * 64), kLds, stream, P);
+    hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT, FEW>), dim3(P.nsplit * P.hk * P.b),
+                       dim3(UnitCfg<BITS, GS, FEW>::NW * 64), kLds, stream, P);
     return hipGetLastError();
+}
+
+// The 4-bit kernels also exist with 8 waves per workgroup that keep six rows in flight each instead of 16 (12)
+// waves with four (P.few_waves, decided on the host).  The prologue, which the waves of a SIMD issue in turn, and
+// the merge of the waves shrink, and a wave's longer run of units hides more latency: 4-7 % faster from 4K to
+// 128K tokens and from 1 to 16 sequences of equal length.  The 16 waves keep more bytes in flight per compute
+// unit, which only pays when a few workgroups are left streaming alone (ragged batches).  A 2-bit unit admits
+// only four rows in flight, and there the 8 waves lose 2-3 %: not built.
+template <int BITS, int GS, bool BF16, bool APPEND, bool KT = false>
+hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
+    if constexpr (few_waves_variant(BITS, GS)) {
+        if (P.few_waves) return launch_fwd_ttt<BITS, GS, BF16, APPEND, KT, true>(P, stream);
+    }
+    return launch_fwd_ttt<BITS, GS, BF16, APPEND, KT, false>(P, stream);
 }
 
 template <int BITS, int GS>

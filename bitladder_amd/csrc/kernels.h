@@ -75,6 +75,7 @@ struct FwdParams {
     // n / nsplit and n / hk as one multiply: magic = ceil(2^32 / d), or 0 for d = 1; exact for n * d < 2^32
     // (a runtime integer division costs the prologue of every workgroup some 100 cycles, and there were five)
     uint32_t nsplit_magic, hk_magic;
+    int few_waves;              // run the 8-wave variant of the kernel (layout.h: few_waves_variant)
 };
 
 inline uint32_t division_magic(uint32_t d) { return d <= 1 ? 0u : static_cast<uint32_t>(((1ull << 32) + d - 1) / d); }

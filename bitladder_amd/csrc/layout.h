@@ -90,4 +90,9 @@ constexpr int decode_waves(int bits, int gs) {
     return unit_region_bytes(bits, gs) <= 9728 ? 16 : (unit_region_bytes(bits, gs) <= 12288 ? 12 : 8);
 }
 
+// The decode kernels that also exist with 8 waves per workgroup (for launches with little work per
+// workgroup), and the number of waves of a launch.
+constexpr bool few_waves_variant(int bits, int gs) { return bits == 4 && decode_waves(bits, gs) > 8; }
+constexpr int kFewWaves = 8;
+
 }  // namespace bitdecode

@@ -119,6 +119,30 @@ def test_decode_many_chunks_per_wave(device, bits, gs):
         assert err < ATOL, (ns, err)
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("gs", [128, 64, 32])
+def test_decode_both_wave_count_variants_of_the_4bit_kernels(device, gs, dtype):
+    """The 4-bit kernels exist with 16 (12 at group 32) and with 8 waves per workgroup; the library takes the
+    8-wave one when a workgroup has at most 16 packed units.  32 units here: one split runs the large variant,
+    two splits the small one with two units per wave (its deeper row pipeline runs on into the second unit),
+    four splits the small one with one unit per wave.  Same bar for all."""
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, S, R, bits = 2, 8, 2, 2048, 40, 4
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=91, dtype=dtype)
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs, dtype=dtype)
+    cache = _pack_gpu(k, v, bits, gs, dtype, device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, want_lse = O.attend_ref(q, k_hat, v_hat, SCALE, k[:, S:], v[:, S:])
+    kres, vres = H.to_dev(k[:, S:], dtype, device), H.to_dev(v[:, S:], dtype, device)
+    tol = H.out_tolerance(want, dtype)
+    for ns in (1, 2, 4):
+        out, lse = fwd_kvcache_int(H.to_dev(q, dtype, device), *cache, None, SCALE, "k-channel", gs, bits,
+                                   k_residual=kres, v_residual=vres, num_splits=ns, return_lse=True)
+        err = np.abs(out.float().cpu().numpy() - want)
+        assert (err <= tol).all(), (ns, err.max())
+        np.testing.assert_allclose(lse.cpu().numpy(), want_lse, atol=2e-3, rtol=1e-4)
+
+
 @pytest.mark.parametrize("bits,gs", [(4, 128), (4, 32), (2, 128), (2, 32)])
 def test_decode_many_splits(device, bits, gs):
     """More splits than one batch of the final merge handles at once (33, 70), and more splits than

@@ -59,7 +59,8 @@ class _Manual:
                 self.k_res[i, r[i]] = k_new[i, 0]
                 self.v_res[i, r[i]] = v_new[i, 0]
         out = fwd_kvcache_int(q, *self.cache, self.table, SCALE, "k-channel", self.gs, self.bits,
-                              seqlens_k=self._i32(p), max_seqlen_k=max(p), k_residual=k_win, v_residual=v_win,
+                              # (the host bound the step uses: the library picks the kernel variant from it)
+                              seqlens_k=self._i32(p), max_seqlen_k=self.capacity, k_residual=k_win, v_residual=v_win,
                               residual_len=self._i32([x + 1 for x in r]), max_residual_len=128, num_splits=ns)
         full = [x == 127 and not o for x, o in zip(r, over)]
         if any(full):
