@@ -107,6 +107,28 @@ def test_step_equals_store_decode_pack(device, bits, gs, dtype, ns):
         assert torch.equal(cache.k_res[i, :r], manual.k_res[i, :r]) and torch.equal(cache.v_res[i, :r], manual.v_res[i, :r])
 
 
+@pytest.mark.parametrize("bits,gs,ns", [(4, 128, 2), (4, 32, 1), (2, 128, 2)])
+def test_step_with_eight_query_heads_per_kv_head(device, bits, gs, ns):
+    """A full GQA group: in the 8-wave kernels every wave of the workgroup merges a head, the two that store the
+    token and count the sequence included."""
+    from bitladder_amd import BitKVCache
+    b, h, h_k, steps, capacity = 2, 8, 1, 140, 512
+    lengths = [250, 5]
+    qs, k, v, qd, kd, vd = _inputs(b, h, h_k, 256 + steps, "fp16", device, 23)
+    cache = BitKVCache(b, h_k, capacity, num_bits=bits, group_size=gs, dtype=torch.float16, device=device)
+    manual = _Manual(b, h_k, capacity, bits, gs, torch.float16, device)
+    cache.prefill(kd[:, :256], vd[:, :256], lengths)
+    manual.prefill(kd[:, :256], vd[:, :256], lengths)
+    for s in range(steps):
+        t = 256 + s
+        out = cache.step(qd[s], kd[:, t:t + 1], vd[:, t:t + 1], SCALE, num_splits=ns)
+        want = manual.step(qd[s], kd[:, t:t + 1], vd[:, t:t + 1], ns)
+        assert torch.equal(out, want), (s, manual.total)
+    assert cache.total.tolist() == manual.total == [x + steps for x in lengths]
+    for got, ref in zip((cache.k_pack, cache.k_params, cache.v_pack, cache.v_params), manual.cache):
+        assert torch.equal(got, ref)
+
+
 def test_step_output_and_packed_window_match_the_oracle(device):
     """The step that fills the window: 128 tokens attended in fp16 behind a quantized prefix, and the chunk it
     leaves in the cache is the oracle's quantization of those 128 tokens."""
