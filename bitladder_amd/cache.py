@@ -18,7 +18,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from .interface import fwd_kvcache_int, kvcache_pack_int, plan_fwd_kvcache_int_append
+from .interface import fwd_kvcache_int, fwd_kvcache_int_append, kvcache_pack_int, plan_fwd_kvcache_int_append
 
 BLOCK = 128          # tokens per packed block = residual window size N_r
 
@@ -141,10 +141,14 @@ class BitKVCache:
             k_new, v_new = k_new[:, None], v_new[:, None]
         if any(p + r + 1 > self.capacity for p, r in zip(self.packed_len, self.res_len)):
             raise ValueError("step: cache capacity exceeded")
-        # (the step's workspace comes from the per-stream cache: nothing is allocated or filled per token)
-        plan = self.plan_step(q, k_new.to(self.dtype), v_new.to(self.dtype), softmax_scale, _stream_ws=True, **kw)
-        with torch.cuda.device(self.device):
-            out = plan.run()
+        if softmax_scale is None:
+            softmax_scale = 1.0 / math.sqrt(q.shape[-1])
+        # (the plain entry point: its workspace comes from the per-stream cache and its argument block is
+        # found again when the same buffers are passed step after step)
+        out = fwd_kvcache_int_append(q, k_new.to(self.dtype), v_new.to(self.dtype), self.k_pack, self.k_params,
+                                     self.v_pack, self.v_params, self.k_res, self.v_res, self.total,
+                                     self.capacity + BLOCK - 1, None, softmax_scale, "k-channel", self.gs, self.bits,
+                                     **kw)
         for i, (p, r) in enumerate(zip(self.packed_len, self.res_len)):
             if r + 1 < BLOCK:
                 self.res_len[i] = r + 1

@@ -73,6 +73,46 @@ def test_dropin_call_reuses_a_per_stream_workspace(device):
     assert np.abs(want.float().cpu().numpy() - ref).max() < 2e-3
 
 
+def test_dropin_call_finds_its_argument_block_again(device):
+    """The plain call keeps the validated argument block of its last few distinct calls.  What must hold: every
+    call returns a tensor of its own, new contents of the same tensors give new results, a call that differs in
+    any tensor's address, strides or type is another call, and nothing keeps the caller's tensors alive."""
+    import gc
+    import weakref
+    from bitladder_amd import fwd_kvcache_int, interface, plan_fwd_kvcache_int
+    q, cache, kr, vr, host = _problem(device, 13)
+    kw = dict(k_residual=kr, v_residual=vr, num_splits=8)
+    args = (None, SCALE, "k-channel", 128, 4)
+    interface._plan_cache().clear()
+    want = plan_fwd_kvcache_int(q, *cache, *args, **kw).run().clone()
+    outs = [fwd_kvcache_int(q, *cache, *args, **kw) for _ in range(4)]
+    assert len(interface._plan_cache()) == 1
+    assert len({o.data_ptr() for o in outs}) == 4 and all(torch.equal(o, want) for o in outs)
+    # the same tensors with new contents
+    q2 = torch.randn_like(q)
+    want2 = plan_fwd_kvcache_int(q2, *cache, *args, **kw).run().clone()
+    q.copy_(q2)
+    out2, lse2 = fwd_kvcache_int(q, *cache, *args, return_lse=True, **kw)          # another call: it returns the LSE
+    out3, lse3 = fwd_kvcache_int(q, *cache, *args, return_lse=True, **kw)          # found again
+    assert torch.equal(out2, want2) and torch.equal(out3, want2) and torch.equal(lse2, lse3)
+    assert lse2.data_ptr() != lse3.data_ptr() and not torch.equal(outs[0], want2)
+    # a strided q of the same contents, and a caller-given output
+    wide = torch.zeros((q.shape[0], 1, q.shape[2], 256), dtype=q.dtype, device=device)
+    wide[..., :128] = q
+    given = torch.empty_like(q)
+    n = len(interface._plan_cache())
+    assert fwd_kvcache_int(wide[..., :128], *cache, *args, out=given, **kw) is given and torch.equal(given, want2)
+    assert len(interface._plan_cache()) == n + 1
+    # an invalid call is still rejected although a valid one over the same cache is held
+    with pytest.raises(RuntimeError):
+        fwd_kvcache_int(q[:, :, :3], *cache, *args, **kw)
+    # the held argument blocks do not hold the caller's tensors
+    ref = weakref.ref(kr)
+    del kr, kw, outs
+    gc.collect()
+    assert ref() is None
+
+
 def test_two_plans_on_two_streams_overlap_without_changing_a_bit(device):
     """Two plans (different problems, a workspace each) replayed many times on two streams at once give,
     every time, the bits they give when run alone."""
