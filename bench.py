@@ -361,9 +361,9 @@ def main():
 
         n_drop = max(50, args.steps)
         result["dropin_eager_us_per_call"] = round(time_steps(dropin, n_drop, 5, False, steady=False)["event_us"], 3)
-        result["dropin_eager_note"] = ("fwd_kvcache_int(...) called %d times in a Python loop, GPU time between first "
-                                       "and last call / calls; bound by the host's per-call work (argument checks, "
-                                       "ctypes), not by the kernel" % n_drop)
+        result["dropin_eager_note"] = ("fwd_kvcache_int(...) called %d times in a Python loop (eager launches), GPU "
+                                       "time between first and last call / calls: the larger of the host's work "
+                                       "per call and the kernel's time" % n_drop)
         assert torch.equal(outs[0], plans[0].run()), "drop-in call and plan disagree"
 
     if not args.no_qpack:
