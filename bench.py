@@ -100,24 +100,13 @@ MIN_TIMED_STEPS = 400      # steps inside the timed region
 WARM_STEPS = 1600          # untimed replayed steps in front of it: the first ~10 ms after idle run 3-10 % slower
 
 
-def slots_needed(steps, warmup, limit):
-    """Smallest number of slots such that, when time_steps(..., steady=True) hands step i to slot i % slots
-    (eager warm-up, capture, every replay of the graph restarting at i = 0), no slot is used more than
-    `limit` times."""
-    nodes = steps * max(1, math.ceil(MIN_GRAPH_NODES / steps))
-    plays = 1 + math.ceil(WARM_STEPS / nodes) + max(1, math.ceil(MIN_TIMED_STEPS / nodes))
-    n = 1
-    while math.ceil(warmup / n) + 1 + plays * math.ceil(nodes / n) > limit:
-        n += 1
-    return n
-
-
-def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True):
+def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True, replay_prologue=None):
     """Times `run_step`.  Eager warm-up of `warmup` steps, then one HIP graph of `nodes` steps (`steps` times
     a whole number, at least MIN_GRAPH_NODES when `steady`) is captured, replayed untimed (once to upload it,
     then for WARM_STEPS steps when `steady`) and replayed `replays` times between two events and two host
     synchronisations.  Without a graph the eager loop runs the same number of steps.  Returns a dict with the
-    wall and event time per step and what was run."""
+    wall and event time per step and what was run.  `replay_prologue`, if given, is captured as the first
+    node(s) of the graph (and called before every `nodes` eager steps): state that the steps advance is reset there."""
     dev = torch.device("cuda:0")
     for i in range(warmup):
         run_step(i)
@@ -135,6 +124,8 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True)
             torch.cuda.current_stream(dev).wait_stream(side)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
+                if replay_prologue is not None:
+                    replay_prologue()
                 for i in range(nodes):
                     run_step(i)
             for _ in range(1 + warm):
@@ -145,6 +136,8 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True)
             graph = None
     if graph is None:
         for i in range(warm * nodes):
+            if replay_prologue is not None and i % nodes == 0:
+                replay_prologue()
             run_step(i)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize(dev)
@@ -155,6 +148,8 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True)
             graph.replay()
     else:
         for i in range(nodes * replays):
+            if replay_prologue is not None and i % nodes == 0:
+                replay_prologue()
             run_step(i)
     e1.record()
     torch.cuda.synchronize(dev)
@@ -402,23 +397,27 @@ def main():
 
     if not args.no_step:
         # the same decode as one launch that also appends the step's new token (device-side lengths).  A slot
-        # is a packed cache with a window and a length counter of its own, starting at S packed tokens + 64 in
-        # the window; there are enough slots that none sees 60 steps (warm-up, capture, untimed and timed
-        # replays together), so no window fills inside the measurement
-        n_slots = max(nbuf, slots_needed(args.steps, args.warmup, 59))
+        # is one of the rotated packed caches with a window and a length counter of its own, S packed tokens + 64
+        # in the window at the start of every graph replay (one small copy node in front of the steps resets the
+        # counters), so that no window fills inside the measurement: a fill is a different, rarer step
+        nodes = args.steps * max(1, math.ceil(MIN_GRAPH_NODES / args.steps))
+        n_slots = max(nbuf, math.ceil((nodes + args.warmup + 1) / 59))
+        start_len = (packed_dev + 64) if ragged else torch.full((b,), S + 64, device=dev)
+        lengths_all = start_len.to(torch.int32).repeat(n_slots, 1).contiguous()
+        lengths_init = lengths_all.clone()
         splans = []
         for i in range(n_slots):
             cache, kres, vres = keep[i % nbuf]
-            lengths = ((packed_dev + 64) if ragged else torch.full((b,), S + 64, device=dev)).to(torch.int32)
             q_t = torch.randn((b, 1, h, 128), device=dev).to(dtype)
             kn = torch.randn((b, 1, h_k, 128), device=dev).to(dtype)
-            splans.append(plan_fwd_kvcache_int_append(q_t, kn, kn.clone(), *cache, kres.clone(), vres.clone(), lengths,
-                                                      S + 127, None, scale, "k-channel", gs, bits,
+            splans.append(plan_fwd_kvcache_int_append(q_t, kn, kn.clone(), *cache, kres.clone(), vres.clone(),
+                                                      lengths_all[i], S + 127, None, scale, "k-channel", gs, bits,
                                                       num_splits=args.num_splits))
-        us_append = time_steps(lambda i: splans[i % n_slots].run(), args.steps, args.warmup, not args.no_graph)["event_us"]
+        us_append = time_steps(lambda i: splans[i % n_slots].run(), args.steps, args.warmup, not args.no_graph,
+                               replay_prologue=lambda: lengths_all.copy_(lengths_init))["event_us"]
         result["decode_step_with_append"] = {
             "entry": "bitdecode_fwd_append", "us_per_step": round(us_append, 3),
-            "window_tokens": "65-123", "does": "attend + store the new token + advance the device-side length"}
+            "window_tokens": "65-%d" % (64 + math.ceil((nodes + args.warmup + 1) / n_slots)), "does": "attend + store the new token + advance the device-side length"}
         del splans
 
     if not args.no_fp16:
