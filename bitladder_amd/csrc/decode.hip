@@ -1051,14 +1051,15 @@ __device__ __forceinline__ float wave_max(float x) {
 __device__ __forceinline__ float2 ld_dev2_at(const float* base, uint32_t lane_bytes) {
     return ld_dev2(reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes));
 }
-// partial outputs (two channels per lane) of splits s0 .. s0+31 of one query head; past the last split the
+// partial outputs (two channels per lane) of splits s0 .. s0+N-1 of one query head; past the last split the
 // last one is read again (its weight is zero)
-__device__ __forceinline__ void load_partials(float2 (&v)[32], const float* head_base, uint32_t lane_bytes,
+template <int N>
+__device__ __forceinline__ void load_partials(float2 (&v)[N], const float* head_base, uint32_t lane_bytes,
                                               uint32_t split_stride, int s0, int nsplit) {
     const float* base = head_base + static_cast<size_t>(s0) * split_stride;
     const int cnt = nsplit - s0;
 #pragma unroll
-    for (int k = 0; k < 32; ++k) {
+    for (int k = 0; k < N; ++k) {
         v[k] = ld_dev2_at(base, lane_bytes);
         base += (k + 1 < cnt) ? split_stride : 0u;
     }
@@ -1066,23 +1067,25 @@ __device__ __forceinline__ void load_partials(float2 (&v)[32], const float* head
 
 // Merge of the splits of one query head by one wave (flash_fwd_kernel.h:1217-1298 in unnormalised
 // form): out = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M).  Lane l owns channels 2l and
-// 2l+1.  Splits are taken 32 at a time: lane l holds the (M, L) pair of split s0 + l % 32, the weights go
-// back to all lanes as scalars.  The order of the additions is fixed.  `split_stride` is in floats and,
-// like the whole partial-output area, below 2^31 bytes (checked by the host).
-__device__ __forceinline__ void merge_splits(const float* o_part, const float* ml_part, int64_t hrow, uint32_t split_stride,
-                                             int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
+// 2l+1.  Splits are taken N at a time (N = 32, or less when there are fewer splits): lane l holds the (M, L) pair of
+// split s0 + l % 32, the weights go back to all lanes as scalars.  The order of the additions is fixed: even
+// and odd splits of a block are summed separately (two dependent chains instead of one) and added at the end.
+// `split_stride` is in floats and, like the whole partial-output area, below 2^31 bytes (checked by the host).
+template <int N>
+__device__ __forceinline__ void merge_splits_n(const float* o_part, const float* ml_part, int64_t hrow, uint32_t split_stride,
+                                               int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
     const float* head_base = o_part + hrow * kHeadDim;
     const float* mlb = ml_part + hrow * nsplit * 2;
     const uint32_t lane_bytes = lane * 8, ml_lane = (lane & 31) * 8;
     const int sl = lane & 31;
     const float2 none = float2{-INFINITY, 0.0f};
-    float2 v[32];
+    float2 v[N];
     float2 ml = none;
     float lacc = 0.0f, Mu = 0.0f;
-    O0 = O1 = 0.0f;
+    float e0 = 0.0f, e1 = 0.0f, d0 = 0.0f, d1 = 0.0f;
     for (int s0 = 0; s0 < nsplit; s0 += 32) {
         if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
-        load_partials(v, head_base, lane_bytes, split_stride, s0, nsplit);
+        load_partials<N>(v, head_base, lane_bytes, split_stride, s0, nsplit);
         if (s0 == 0) {
             float mx = ml.x;
             for (int s = 32; s < nsplit; s += 32) {        // more than 32 splits: the other maxima
@@ -1094,15 +1097,33 @@ __device__ __forceinline__ void merge_splits(const float* o_part, const float* m
         const float w = (s0 + sl < nsplit) ? __builtin_amdgcn_exp2f(ml.x - Mu) : 0.0f;
         lacc = __builtin_fmaf(w, ml.y, lacc);
 #pragma unroll
-        for (int k = 0; k < 32; ++k) {
-            const float wk = lane_value(w, k);
-            O0 = __builtin_fmaf(wk, v[k].x, O0);
-            O1 = __builtin_fmaf(wk, v[k].y, O1);
+        for (int k = 0; k < N; k += 2) {
+            const float wa = lane_value(w, k), wb = lane_value(w, k + 1);
+            e0 = __builtin_fmaf(wa, v[k].x, e0);
+            e1 = __builtin_fmaf(wa, v[k].y, e1);
+            d0 = __builtin_fmaf(wb, v[k + 1].x, d0);
+            d1 = __builtin_fmaf(wb, v[k + 1].y, d1);
         }
     }
+    O0 = e0 + d0;
+    O1 = e1 + d1;
     // both halves of the wave hold the same 32 terms
     const float lrow = row_sum16(lacc);
     L = lane_value(lrow, 0) + lane_value(lrow, 16);
+}
+__device__ __forceinline__ void merge_splits(const float* o_part, const float* ml_part, int64_t hrow, uint32_t split_stride,
+                                             int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
+    // as many loads per lane as there are splits, rounded up to 4, 8, 16 or 32: every one of them is a round trip
+    // of its own to the memory side (with 32 loads for 8 splits the 4K-token step took 0.5 us longer)
+    if (nsplit <= 4) {
+        merge_splits_n<4>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+    } else if (nsplit <= 8) {
+        merge_splits_n<8>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+    } else if (nsplit <= 16) {
+        merge_splits_n<16>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+    } else {
+        merge_splits_n<32>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+    }
 }
 
 template <bool BF16>
