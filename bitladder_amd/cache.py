@@ -32,16 +32,25 @@ class BitKVCache:
     """
 
     def __init__(self, batch: int, kv_heads: int, max_tokens: int, *, num_bits: int = 4, group_size: int = 128,
-                 dtype: torch.dtype = torch.float16, device="cuda", head_dim: int = 128):
+                 dtype: torch.dtype = torch.float16, device="cuda", head_dim: int = 128,
+                 quant_mode: str = "k-channel"):
         if head_dim != 128:
             raise NotImplementedError("head_dim must be 128")
+        if quant_mode not in ("k-channel", "k-tensor"):
+            raise ValueError(f"quant_mode must be 'k-channel' or 'k-tensor', got {quant_mode!r}")
+        if quant_mode == "k-tensor" and num_bits != 4:
+            raise NotImplementedError("quant_mode 'k-tensor' is implemented for num_bits=4 only")
         self.b, self.h_k, self.bits, self.gs, self.dtype = batch, kv_heads, num_bits, group_size, dtype
+        self.quant_mode = quant_mode
         self.device = torch.device(device)
         self.capacity = (max_tokens + BLOCK - 1) // BLOCK * BLOCK
         pn, S, d = 16 // num_bits, self.capacity, head_dim
         dev = self.device
         self.k_pack = torch.zeros((batch, S // pn, kv_heads, d), dtype=torch.uint16, device=dev)
-        self.k_params = torch.zeros((batch, S // group_size, kv_heads, d), dtype=torch.float32, device=dev)
+        # "k-tensor": one (scale, zero) per token and channel group for K as well, shaped like V's
+        k_params_shape = (batch, d // group_size, kv_heads, S) if quant_mode == "k-tensor" \
+            else (batch, S // group_size, kv_heads, d)
+        self.k_params = torch.zeros(k_params_shape, dtype=torch.float32, device=dev)
         self.v_pack = torch.zeros((batch, S, kv_heads, d // pn), dtype=torch.uint16, device=dev)
         self.v_params = torch.zeros((batch, d // group_size, kv_heads, S), dtype=torch.float32, device=dev)
         self.k_res = torch.zeros((batch, BLOCK, kv_heads, d), dtype=dtype, device=dev)
@@ -77,7 +86,7 @@ class BitKVCache:
             # sequences shorter than n_pack get blocks of padding packed behind their prefix; decode never
             # reads them (seqlens_k) and later appends overwrite them
             kvcache_pack_int(k[:, :n_pack], self.k_pack, self.k_params, v[:, :n_pack], self.v_pack, self.v_params,
-                             None, None, n_pack, "k-channel", self.gs, self.bits)
+                             None, None, n_pack, self.quant_mode, self.gs, self.bits)
         for i, (p, r) in enumerate(zip(self.packed_len, self.res_len)):
             if r:
                 self.k_res[i, :r].copy_(k[i, p:p + r])
@@ -100,7 +109,7 @@ class BitKVCache:
             full = [r == BLOCK for r in self.res_len]
             offsets = self._i32([p if f else -1 for p, f in zip(self.packed_len, full)])
             kvcache_pack_int(self.k_res, self.k_pack, self.k_params, self.v_res, self.v_pack, self.v_params,
-                             None, None, BLOCK, "k-channel", self.gs, self.bits, dst_offsets=offsets)
+                             None, None, BLOCK, self.quant_mode, self.gs, self.bits, dst_offsets=offsets)
             self.packed_len = [p + BLOCK if f else p for p, f in zip(self.packed_len, full)]
             self.res_len = [0 if f else r for r, f in zip(self.res_len, full)]
         self.total += 1
@@ -112,7 +121,7 @@ class BitKVCache:
             softmax_scale = 1.0 / math.sqrt(q.shape[-1])
         max_p, max_r = max(self.packed_len), max(self.res_len)
         return fwd_kvcache_int(q, self.k_pack, self.k_params, self.v_pack, self.v_params, None, softmax_scale,
-                               "k-channel", self.gs, self.bits,
+                               self.quant_mode, self.gs, self.bits,
                                seqlens_k=self._i32(self.packed_len), max_seqlen_k=max_p,
                                k_residual=self.k_res, v_residual=self.v_res,
                                residual_len=self._i32(self.res_len), max_residual_len=max_r, **kw)
@@ -130,7 +139,7 @@ class BitKVCache:
             softmax_scale = 1.0 / math.sqrt(q.shape[-1])
         return plan_fwd_kvcache_int_append(q, k_new, v_new, self.k_pack, self.k_params, self.v_pack, self.v_params,
                                            self.k_res, self.v_res, self.total, self.capacity + BLOCK - 1, None,
-                                           softmax_scale, "k-channel", self.gs, self.bits, **kw)
+                                           softmax_scale, self.quant_mode, self.gs, self.bits, **kw)
 
     def step(self, q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
              softmax_scale: Optional[float] = None, **kw) -> torch.Tensor:
@@ -147,7 +156,7 @@ class BitKVCache:
         # found again when the same buffers are passed step after step)
         out = fwd_kvcache_int_append(q, k_new.to(self.dtype), v_new.to(self.dtype), self.k_pack, self.k_params,
                                      self.v_pack, self.v_params, self.k_res, self.v_res, self.total,
-                                     self.capacity + BLOCK - 1, None, softmax_scale, "k-channel", self.gs, self.bits,
+                                     self.capacity + BLOCK - 1, None, softmax_scale, self.quant_mode, self.gs, self.bits,
                                      **kw)
         for i, (p, r) in enumerate(zip(self.packed_len, self.res_len)):
             if r + 1 < BLOCK:

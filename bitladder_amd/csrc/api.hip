@@ -50,13 +50,11 @@ int check_quant(int bits, int gs, int dtype, int d) {
     return 0;
 }
 
-int check_mode(int quant_mode, int bits, bool step) {
+int check_mode(int quant_mode, int bits) {
     if (quant_mode != BITDECODE_K_CHANNEL && quant_mode != BITDECODE_K_TENSOR)
         return fail(BITDECODE_EINVAL, "quant_mode %d (k-channel=0, k-tensor=1)", quant_mode);
     if (quant_mode == BITDECODE_K_TENSOR && bits != 4)
         return fail(BITDECODE_EUNSUPPORTED, "quant_mode k-tensor is implemented for 4 bits only (as in the reference)");
-    if (quant_mode == BITDECODE_K_TENSOR && step)
-        return fail(BITDECODE_EUNSUPPORTED, "the decode step with append is not implemented for quant_mode k-tensor");
     return 0;
 }
 
@@ -128,7 +126,7 @@ int bitdecode_qpack(const bitdecode_qpack_args* a, void* stream) {
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
     if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
-    if (int rc = check_mode(a->quant_mode, a->bits, false)) return rc;
+    if (int rc = check_mode(a->quant_mode, a->bits)) return rc;
     if (a->b < 0 || a->h_k <= 0 || a->n_tokens < 0) return fail(BITDECODE_EINVAL, "negative size");
     if (a->n_tokens % kChunk) return fail(BITDECODE_EINVAL, "n_tokens %d is not a multiple of 128", a->n_tokens);
     if (a->cache_tokens % kChunk || a->cache_tokens <= 0)
@@ -199,7 +197,7 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     using namespace bitdecode;
     if (!a) return fail(BITDECODE_EINVAL, "args is null");
     if (int rc = check_quant(a->bits, a->group_size, a->dtype, a->d)) return rc;
-    if (int rc = check_mode(a->quant_mode, a->bits, step != nullptr)) return rc;
+    if (int rc = check_mode(a->quant_mode, a->bits)) return rc;
     if (a->b <= 0 || a->h <= 0 || a->h_k <= 0) return fail(BITDECODE_EINVAL, "batch and head counts must be positive");
     if (a->h % a->h_k) return fail(BITDECODE_EINVAL, "h %d is not a multiple of h_k %d", a->h, a->h_k);
     const int g = a->h / a->h_k;

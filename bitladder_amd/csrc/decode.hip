@@ -1213,7 +1213,7 @@ __device__ __forceinline__ void step_begin(int bi, int hk, int t) {
 // Second part, by the whole workgroup once the output is written: a window that the token filled is
 // quantize-packed (127 rows from the window, the last one from the new-token tensors) into the chunk
 // behind the packed prefix.  `lds` is the workgroup's whole dynamic LDS.
-template <int BITS, int GS, bool BF16>
+template <int BITS, int GS, bool BF16, bool KT>
 __device__ __forceinline__ void step_end(uint8_t* lds, int bi, int hk, int t) {
     const int tid = threadIdx.x;
     const int r = t & (kChunk - 1), packed = t - r;
@@ -1227,11 +1227,11 @@ __device__ __forceinline__ void step_end(uint8_t* lds, int bi, int hk, int t) {
         const int64_t k_st = LATE_I64(kres_st), v_st = LATE_I64(vres_st);
         const ChunkPlace place = chunk_place(LATE_PTR(const int*, block_table), LATE_I64(bt_stride),
                                              LATE_I32(chunks_per_page), bi, hk, LATE_I32(hk), packed / kChunk);
-        const qp::ChunkDst D = qp::chunk_dst<BITS, GS>(
+        const qp::ChunkDst D = qp::chunk_dst<BITS, GS, KT>(
             LATE_PTR(uint8_t*, k_pack), LATE_PTR(uint8_t*, k_params), LATE_PTR(uint8_t*, v_pack),
             LATE_PTR(uint8_t*, v_params), LATE_I64(kpack_bh), LATE_I64(kparams_bh), LATE_I64(vpack_bh),
             LATE_I64(vparams_bh), place);
-        qp::pack_chunk<BITS, GS, BF16, false>(
+        qp::pack_chunk<BITS, GS, BF16, false, KT>(
             *reinterpret_cast<qp::PackLds<GS>*>(lds), tid, tid < qp::kPackThreads,
             [=](int n) { return n == kChunk - 1 ? kn : kw + n * k_st; },
             [=](int n) { return n == kChunk - 1 ? vn : vw + n * v_st; }, D);
@@ -1258,7 +1258,7 @@ constexpr int fwd_lds_bytes() {
 
 template <int BITS, int GS, bool BF16, bool APPEND, bool KT, bool FEW>
 __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
-    static_assert(!KT || (BITS == 4 && !APPEND), "per-token K parameters: 4 bits, plain decode");
+    static_assert(!KT || BITS == 4, "per-token K parameters: 4 bits");
     using C = UnitCfg<BITS, GS, FEW>;
     constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -1528,7 +1528,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }
-        if (appends) step_end<BITS, GS, BF16>(lds, bi, hk, step_len);
+        if (appends) step_end<BITS, GS, BF16, KT>(lds, bi, hk, step_len);
     }
     PROF(7);
     PROF_FLUSH();
@@ -1569,9 +1569,12 @@ hipError_t launch_fwd_tt(const FwdParams& P, hipStream_t stream) {
 
 template <int BITS, int GS>
 hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
-    if (P.ktensor) {      // "k-tensor" mode: 4 bits, plain decode
+    if (P.ktensor) {      // "k-tensor" mode: 4 bits
         if constexpr (BITS == 4) {
-            if (P.lengths) return hipErrorInvalidValue;
+            if (P.lengths) {
+                return P.bf16 ? launch_fwd_tt<BITS, GS, true, true, true>(P, stream)
+                              : launch_fwd_tt<BITS, GS, false, true, true>(P, stream);
+            }
             return P.bf16 ? launch_fwd_tt<BITS, GS, true, false, true>(P, stream)
                           : launch_fwd_tt<BITS, GS, false, false, true>(P, stream);
         } else {

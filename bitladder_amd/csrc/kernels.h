@@ -57,7 +57,7 @@ struct FwdParams {
     int xcd_remap;             // (b * hk) % 8 == 0: keep the splits of one (batch, kv-head) on one XCD
     int neg_scale;             // softmax_scale < 0: the sign is folded into q
     int bits, gs, bf16;
-    int ktensor;                // "k-tensor" mode, as in QpackParams (4 bits, no append)
+    int ktensor;                // "k-tensor" mode, as in QpackParams (4 bits)
     const int* block_table;     // paged cache, as in QpackParams
     int64_t bt_stride;
     int chunks_per_page;

@@ -481,8 +481,6 @@ def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: tor
                                 return_lse: bool = False,
                                 _stream_ws: bool = False) -> DecodePlan:
     """Validates a decode step with append and returns its `DecodePlan`; see `fwd_kvcache_int_append`."""
-    if quant_mode == "k-tensor":
-        raise NotImplementedError("the decode step with append is not implemented for quant_mode 'k-tensor'")
     if k_residual is None or v_residual is None or k_residual.dim() != 4 or k_residual.shape[1] < CHUNK:
         raise RuntimeError(f"the residual window must hold at least {CHUNK} tokens")
     max_len = int(max_len)

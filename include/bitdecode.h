@@ -35,7 +35,7 @@ enum { BITDECODE_FP16 = 0, BITDECODE_BF16 = 1 };
  * groups of tokens ("k-channel"), or per token over groups of channels like V ("k-tensor":
  * csrc/bit_decode/src/include/qpack.h:378-470, dequantize.h:403-475; its dispatch is commented out in the
  * reference, decode_api.cpp:195-203, 217-225).  "k-tensor" is implemented for 4 bits, as in the reference,
- * and not for bitdecode_fwd_append; k_params then has v_params' shape. */
+ * in every entry point; k_params then has v_params' shape. */
 enum { BITDECODE_K_CHANNEL = 0, BITDECODE_K_TENSOR = 1 };
 
 /* Quantize-pack n_tokens new tokens of K and V into the packed cache.

@@ -80,13 +80,12 @@ def test_pack_then_decode_ktensor_ragged_with_window(device, dtype, gs):
         assert (diff < H.out_tolerance(want, dtype, ATOL)).all(), (dtype, gs, ns, diff.max())
 
 
-def test_ktensor_is_rejected_where_it_is_not_implemented(device):
+def test_ktensor_is_rejected_at_two_bits(device):
     from bitladder_amd import fwd_kvcache_int_append, kvcache_pack_int
     t = torch.zeros(1, 128, 2, 128, dtype=torch.float16, device=device)
     cache = H.alloc_cache(1, 128, 2, 2, 128, device, k_tensor=True)
     with pytest.raises(NotImplementedError):
         kvcache_pack_int(t, cache[0], cache[1], t, cache[2], cache[3], None, None, 128, "k-tensor", 128, 2)
-    cache = H.alloc_cache(1, 128, 2, 4, 128, device, k_tensor=True)
     with pytest.raises(NotImplementedError):
         fwd_kvcache_int_append(t[:, :1], t[:, :1], t[:, :1], *cache, t, t, torch.zeros(1, dtype=torch.int32, device=device),
-                               128, None, 1.0, "k-tensor", 128, 4)
+                               0, None, 1.0, "k-tensor", 128, 2)

@@ -20,10 +20,13 @@ SCALE = 1.0 / math.sqrt(128)
 class _Manual:
     """The step spelled out with the plain entry points, lengths kept on the host."""
 
-    def __init__(self, b, h_k, capacity, bits, gs, dtype, device, table=None, pool_pages=0, page=0):
+    def __init__(self, b, h_k, capacity, bits, gs, dtype, device, table=None, pool_pages=0, page=0,
+                 quant_mode="k-channel"):
         self.b, self.bits, self.gs, self.device, self.table = b, bits, gs, device, table
-        self.cache = (H.alloc_cache(pool_pages, page, h_k, bits, gs, device) if table is not None
-                      else H.alloc_cache(b, capacity, h_k, bits, gs, device))
+        self.mode = quant_mode
+        kt = quant_mode == "k-tensor"
+        self.cache = (H.alloc_cache(pool_pages, page, h_k, bits, gs, device, k_tensor=kt) if table is not None
+                      else H.alloc_cache(b, capacity, h_k, bits, gs, device, k_tensor=kt))
         self.k_res = torch.zeros((b, 128, h_k, 128), dtype=dtype, device=device)
         self.v_res = torch.zeros_like(self.k_res)
         self.capacity = capacity
@@ -34,7 +37,7 @@ class _Manual:
         n_pack = max(lengths) // 128 * 128
         if n_pack:
             kvcache_pack_int(k[:, :n_pack], self.cache[0], self.cache[1], v[:, :n_pack], self.cache[2], self.cache[3],
-                             self.table, None, n_pack, "k-channel", self.gs, self.bits)
+                             self.table, None, n_pack, self.mode, self.gs, self.bits)
         for i, L in enumerate(lengths):
             p = L // 128 * 128
             self.k_res[i, :L - p] = k[i, p:L]
@@ -58,14 +61,14 @@ class _Manual:
             if not over[i] and k_win is not self.k_res:
                 self.k_res[i, r[i]] = k_new[i, 0]
                 self.v_res[i, r[i]] = v_new[i, 0]
-        out = fwd_kvcache_int(q, *self.cache, self.table, SCALE, "k-channel", self.gs, self.bits,
+        out = fwd_kvcache_int(q, *self.cache, self.table, SCALE, self.mode, self.gs, self.bits,
                               # (the host bound the step uses: the library picks the kernel variant from it)
                               seqlens_k=self._i32(p), max_seqlen_k=self.capacity, k_residual=k_win, v_residual=v_win,
                               residual_len=self._i32([x + 1 for x in r]), max_residual_len=128, num_splits=ns)
         full = [x == 127 and not o for x, o in zip(r, over)]
         if any(full):
             kvcache_pack_int(self.k_res, self.cache[0], self.cache[1], self.v_res, self.cache[2], self.cache[3],
-                             self.table, None, 128, "k-channel", self.gs, self.bits,
+                             self.table, None, 128, self.mode, self.gs, self.bits,
                              dst_offsets=self._i32([y if f else -1 for y, f in zip(p, full)]))
         self.total = [t if o else t + 1 for t, o in zip(self.total, over)]
         return out
@@ -129,31 +132,54 @@ def test_step_with_eight_query_heads_per_kv_head(device, bits, gs, ns):
         assert torch.equal(got, ref)
 
 
-def test_step_output_and_packed_window_match_the_oracle(device):
+@pytest.mark.parametrize("gs,dtype,ns", [(128, "fp16", 2), (64, "bf16", 1), (32, "fp16", 3)])
+def test_step_with_k_quantized_per_token(device, gs, dtype, ns):
+    """quant_mode "k-tensor" through the one-launch step: the same composition, with K's parameters per token."""
+    from bitladder_amd import BitKVCache
+    b, h, h_k, steps, capacity, bits = 3, 8, 2, 140, 640, 4
+    lengths = [120, 255, 0]
+    tdt = H.torch_dtype(dtype)
+    qs, k, v, qd, kd, vd = _inputs(b, h, h_k, 256 + steps, dtype, device, 31)
+    cache = BitKVCache(b, h_k, capacity, num_bits=bits, group_size=gs, dtype=tdt, device=device, quant_mode="k-tensor")
+    manual = _Manual(b, h_k, capacity, bits, gs, tdt, device, quant_mode="k-tensor")
+    cache.prefill(kd[:, :256], vd[:, :256], lengths)
+    manual.prefill(kd[:, :256], vd[:, :256], lengths)
+    for s in range(steps):
+        t = 256 + s
+        out = cache.step(qd[s], kd[:, t:t + 1], vd[:, t:t + 1], SCALE, num_splits=ns)
+        want = manual.step(qd[s], kd[:, t:t + 1], vd[:, t:t + 1], ns)
+        assert torch.equal(out, want), (s, manual.total)
+    assert cache.total.tolist() == manual.total == [x + steps for x in lengths]
+    for got, ref in zip((cache.k_pack, cache.k_params, cache.v_pack, cache.v_params), manual.cache):
+        assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("mode", ["k-channel", "k-tensor"])
+def test_step_output_and_packed_window_match_the_oracle(device, mode):
     """The step that fills the window: 128 tokens attended in fp16 behind a quantized prefix, and the chunk it
     leaves in the cache is the oracle's quantization of those 128 tokens."""
     from bitladder_amd import fwd_kvcache_int_append, kvcache_pack_int
     b, h, h_k, bits, gs, S = 2, 8, 2, 4, 128, 256
     q, k, v = O.make_inputs(b, h, h_k, S + 128, 0, seed=29)
     qd, kd, vd = H.to_dev(q, "fp16", device), H.to_dev(k, "fp16", device), H.to_dev(v, "fp16", device)
-    cache = H.alloc_cache(b, S + 128, h_k, bits, gs, device)
-    kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S, "k-channel", gs, bits)
+    cache = H.alloc_cache(b, S + 128, h_k, bits, gs, device, k_tensor=mode == "k-tensor")
+    kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S, mode, gs, bits)
     k_res = kd[:, S:S + 128].clone()
     v_res = vd[:, S:S + 128].clone()
     k_res[:, 127] = 0          # the last row arrives as the new token
     v_res[:, 127] = 0
     lengths = torch.full((b,), S + 127, dtype=torch.int32, device=device)
     out, lse = fwd_kvcache_int_append(qd, kd[:, S + 127:], vd[:, S + 127:], *cache, k_res, v_res, lengths, S + 127,
-                                      None, SCALE, "k-channel", gs, bits, return_lse=True)
+                                      None, SCALE, mode, gs, bits, return_lse=True)
     torch.cuda.synchronize()
     assert lengths.tolist() == [S + 128] * b
     assert torch.equal(k_res, kd[:, S:S + 128]) and torch.equal(v_res, vd[:, S:S + 128])
-    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs)
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs, quant_mode=mode)
     k_hat, v_hat = O.dequantize_ref(qkv)
     ref, ref_lse = O.attend_ref(q, k_hat, v_hat, SCALE, k[:, S:], v[:, S:])
     assert np.abs(out.float().cpu().numpy() - ref).max() < 2e-3
     assert np.abs(lse.cpu().numpy() - ref_lse).max() < 2e-3
-    H.assert_cache_equals_oracle(H.cache_to_numpy(*cache), O.quantize_kv_ref(k, v, bits, gs))
+    H.assert_cache_equals_oracle(H.cache_to_numpy(*cache), O.quantize_kv_ref(k, v, bits, gs, quant_mode=mode))
 
 
 def test_step_leaves_a_full_sequence_unchanged(device):

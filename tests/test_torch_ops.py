@@ -98,3 +98,39 @@ def test_operators_equal_the_plain_functions_also_when_compiled(device):
     bb = ops.fwd_kvcache_int_append(qd, kn, vn, *c1, k1, v1, l1, S + R, None, SCALE, gs, bits, 2)
     assert torch.equal(a, bb) and torch.equal(l0, l1) and torch.equal(k0, k1) and torch.equal(v0, v1)
     assert l1.tolist() == [S + R + 1] * b
+
+
+@pytest.mark.gpu
+def test_operators_pass_the_quantization_mode_on(device):
+    """`quant_mode` is the last argument of each operator: "k-tensor" gives what the plain functions give."""
+    import bitladder_amd.torch_ops  # noqa: F401
+    from bitladder_amd import fwd_kvcache_int, fwd_kvcache_int_append, kvcache_pack_int
+    from oracle import bitdecode_oracle as O
+    b, h, h_k, S, bits, gs, mode = 2, 8, 2, 256, 4, 64, "k-tensor"
+    q, k, v = O.make_inputs(b, h, h_k, S + 1, 0, seed=19)
+    qd, kd, vd = H.to_dev(q, "fp16", device), H.to_dev(k, "fp16", device), H.to_dev(v, "fp16", device)
+    ops = torch.ops.bitladder_amd
+    caches = [H.alloc_cache(b, S + 128, h_k, bits, gs, device, k_tensor=True) for _ in range(2)]
+    kvcache_pack_int(kd[:, :S], caches[0][0], caches[0][1], vd[:, :S], caches[0][2], caches[0][3], None, None, S,
+                     mode, gs, bits)
+    ops.kvcache_pack_int(kd[:, :S], caches[1][0], caches[1][1], vd[:, :S], caches[1][2], caches[1][3], None, gs, bits,
+                         quant_mode=mode)
+    for g_, w_ in zip(caches[1], caches[0]):
+        assert torch.equal(g_, w_)
+    held = torch.full((b,), S, dtype=torch.int32, device=device)
+    want = fwd_kvcache_int(qd, *caches[0], None, SCALE, mode, gs, bits, seqlens_k=held, max_seqlen_k=S, num_splits=2)
+    got = ops.fwd_kvcache_int(qd, *caches[1], None, SCALE, gs, bits, held, S, num_splits=2, quant_mode=mode)
+    assert torch.equal(got, want)
+    outs = []
+    for i, cache in enumerate(caches):
+        win_k = torch.zeros((b, 128, h_k, 128), dtype=torch.float16, device=device)
+        win_v = torch.zeros_like(win_k)
+        lengths = torch.full((b,), S, dtype=torch.int32, device=device)
+        if i == 0:
+            outs.append(fwd_kvcache_int_append(qd, kd[:, S:], vd[:, S:], *cache, win_k, win_v, lengths, S, None, SCALE,
+                                               mode, gs, bits, num_splits=2))
+        else:
+            outs.append(ops.fwd_kvcache_int_append(qd, kd[:, S:], vd[:, S:], *cache, win_k, win_v, lengths, S, None,
+                                                   SCALE, gs, bits, 2, quant_mode=mode))
+        assert lengths.tolist() == [S + 1] * b
+    assert torch.equal(outs[0], outs[1])
