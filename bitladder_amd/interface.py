@@ -156,12 +156,15 @@ def _split_plan(dev_index, b, h, h_k, max_seqlen, max_res, new_tokens, bits, gs,
     return hit
 
 
-_MAX_PLANS = 8
+# A decode loop over a model makes one distinct call per attention layer and token, each over its layer's own
+# cache: the kept argument blocks must cover all layers (a block is a few hundred bytes plus a reference to
+# the stream's shared workspace), or every call of the loop would miss.
+_MAX_PLANS = 512
 _tls = threading.local()
 
 
 def _plan_cache() -> dict:
-    """Argument blocks of this thread's last few distinct drop-in calls (a thread of its own each: a block is
+    """Argument blocks of this thread's last distinct drop-in calls (a thread of its own each: a block is
     patched with the call's output pointer before it is handed to the library)."""
     c = getattr(_tls, "plans", None)
     if c is None:
@@ -185,7 +188,7 @@ def _call_key(tensors, scalars, kwargs):
 
 def _run_kept(key, q, kwargs, make_plan):
     """Runs a plain (non-plan) decode call.  A decode loop makes such a call again and again over the same
-    memory: the validated argument block of a thread's last few distinct calls is kept and found again by the
+    memory: the validated argument block of a thread's last distinct calls (up to 512) is kept and found again by the
     address, shape, strides and element type of every tensor, which saves 40 % of the host's time per call."""
     return_lse = kwargs.get("return_lse", False)
     cache = _plan_cache()

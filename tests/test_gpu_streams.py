@@ -113,6 +113,26 @@ def test_dropin_call_finds_its_argument_block_again(device):
     assert ref() is None
 
 
+def test_dropin_calls_of_a_whole_model_keep_their_argument_blocks(device):
+    """A decode loop makes one call per attention layer and token, each over that layer's cache: the calls of
+    all layers of a deep model are kept side by side, so the second token's calls find theirs again."""
+    from bitladder_amd import fwd_kvcache_int, interface, plan_fwd_kvcache_int
+    layers = 80
+    q, cache0, kr, vr, _ = _problem(device, 17, S=256)
+    caches = [cache0] + [tuple(t.clone() for t in cache0) for _ in range(layers - 1)]
+    for i, c in enumerate(caches):
+        c[1].view(torch.float16)[..., :128].mul_(1.0 + i / 64.0)      # each layer its own K scales
+    args = (None, SCALE, "k-channel", 128, 4)
+    kw = dict(k_residual=kr, v_residual=vr, num_splits=2)
+    wants = [plan_fwd_kvcache_int(q, *c, *args, **kw).run().clone() for c in caches]
+    assert not torch.equal(wants[0], wants[1])
+    interface._plan_cache().clear()
+    for token in range(3):
+        for c, want in zip(caches, wants):
+            assert torch.equal(fwd_kvcache_int(q, *c, *args, **kw), want)
+        assert len(interface._plan_cache()) == layers
+
+
 def test_two_plans_on_two_streams_overlap_without_changing_a_bit(device):
     """Two plans (different problems, a workspace each) replayed many times on two streams at once give,
     every time, the bits they give when run alone."""
