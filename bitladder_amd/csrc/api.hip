@@ -106,7 +106,7 @@ static size_t ticket_bytes(int32_t b, int32_t h) { return static_cast<size_t>(b)
 
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     if (num_splits <= 1) return 0;
-    return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kHeadDim + 2) * sizeof(float);
+    return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kPartialWords + 2) * sizeof(float);
 }
 
 // paged cache: cache_tokens is the page size; the table must cover `tokens` per sequence
@@ -250,7 +250,7 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
     if (nsplit > 512) return fail(BITDECODE_EINVAL, "num_splits %d is above the limit of 512", nsplit);
     if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
-    if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim * sizeof(float) >= (size_t(1) << 31))
+    if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords * sizeof(uint32_t) >= (size_t(1) << 31))
         return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d heads: partial outputs of 2 GiB or more", nsplit, a->b, a->h);
     // the kernel divides workgroup ids and unit counts by the split count and the head count with a
     // multiply (kernels.h: division_magic), exact while numerator x divisor stays below 2^32
@@ -262,7 +262,7 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     }
     if (static_scratch) {
         const size_t rows = static_cast<size_t>(a->b) * a->h;
-        const size_t need = nsplit > 1 ? static_cast<size_t>(nsplit) * rows * (kHeadDim + 2) * sizeof(float) : 0;
+        const size_t need = nsplit > 1 ? static_cast<size_t>(nsplit) * rows * (kPartialWords + 2) * sizeof(float) : 0;
         if (rows > kStaticHeads || need > kStaticScratchBytes - kStaticCounterBytes)
             return fail(BITDECODE_EWORKSPACE, "bitdecode_fwd_static: %d splits x %zu (batch x head) rows need %zu bytes; the "
                         "built-in scratch holds %zu rows and %zu bytes (use bitdecode_fwd with a workspace)", nsplit, rows,
@@ -337,12 +337,12 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     }
     if (nsplit > 1 && static_scratch) {
         P.tickets = reinterpret_cast<int*>(static_scratch);
-        P.o_part = reinterpret_cast<float*>(static_scratch + kStaticCounterBytes);
-        P.ml_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
+        P.o_part = reinterpret_cast<uint32_t*>(static_scratch + kStaticCounterBytes);
+        P.ml_part = reinterpret_cast<float*>(P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords);
     } else if (nsplit > 1) {
         P.tickets = reinterpret_cast<int*>(ws);
-        P.o_part = reinterpret_cast<float*>(ws + ticket_bytes(a->b, a->h));
-        P.ml_part = P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kHeadDim;
+        P.o_part = reinterpret_cast<uint32_t*>(ws + ticket_bytes(a->b, a->h));
+        P.ml_part = reinterpret_cast<float*>(P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords);
     }
     hipError_t e = launch_fwd(P, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));

@@ -1017,6 +1017,26 @@ __device__ __forceinline__ float2 ld_dev2(const float* p) {
     return float2{__uint_as_float(static_cast<uint32_t>(bits)), __uint_as_float(static_cast<uint32_t>(bits >> 32))};
 }
 
+// the same for 4 bytes
+__device__ __forceinline__ void st_dev1(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t ld_dev1_at(const uint32_t* base, uint32_t lane_bytes) {
+    return __hip_atomic_load(reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// A split's partial output as it crosses workgroups: normalised (O / L: a weighted mean of V rows, so inside the
+// value range of V whatever the split's length) and rounded to nearest fp16, two channels per 32-bit word.
+// Half the bytes of fp32 partials: the workgroup that merges reads g x splits of them through one compute
+// unit's memory path, which is what its time goes into (32 splits of 4 heads: 0.45 us less per step).
+__device__ __forceinline__ uint32_t pack_partial(float O0, float O1, float L) {
+    const float inv = L > 0.0f ? __builtin_amdgcn_rcpf(L) : 0.0f;
+    const _Float16 a = static_cast<_Float16>(O0 * inv), b = static_cast<_Float16>(O1 * inv);
+    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, a)) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, b)) << 16);
+}
+__device__ __forceinline__ float partial_lo(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w))); }
+__device__ __forceinline__ float partial_hi(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16))); }
+
 // x of lane `l` (wave-uniform index) as a scalar
 __device__ __forceinline__ float lane_value(float x, int l) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l));
@@ -1051,41 +1071,45 @@ __device__ __forceinline__ float wave_max(float x) {
 __device__ __forceinline__ float2 ld_dev2_at(const float* base, uint32_t lane_bytes) {
     return ld_dev2(reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes));
 }
-// partial outputs (two channels per lane) of splits s0 .. s0+N-1 of one query head; past the last split the
-// last one is read again (its weight is zero)
+// partial outputs (two channels per lane, 4 bytes) of splits s0 .. s0+N-1 of one query head.  The splits of a
+// head lie 256 bytes apart, so a full block of N loads differs only in the instruction's immediate offset and is
+// issued back to back; past the last split the last one is read again (its weight is zero).
 template <int N>
-__device__ __forceinline__ void load_partials(float2 (&v)[N], const float* head_base, uint32_t lane_bytes,
-                                              uint32_t split_stride, int s0, int nsplit) {
-    const float* base = head_base + static_cast<size_t>(s0) * split_stride;
+__device__ __forceinline__ void load_partials(uint32_t (&v)[N], const uint32_t* head_base, uint32_t lane_bytes,
+                                              int s0, int nsplit) {
+    const uint32_t* base = head_base + s0 * kPartialWords;
     const int cnt = nsplit - s0;
+    if (cnt >= N) {
 #pragma unroll
-    for (int k = 0; k < N; ++k) {
-        v[k] = ld_dev2_at(base, lane_bytes);
-        base += (k + 1 < cnt) ? split_stride : 0u;
+        for (int k = 0; k < N; ++k) v[k] = ld_dev1_at(base + k * kPartialWords, lane_bytes);
+    } else {
+#pragma unroll
+        for (int k = 0; k < N; ++k) v[k] = ld_dev1_at(base + (k < cnt ? k : cnt - 1) * kPartialWords, lane_bytes);
     }
 }
 
-// Merge of the splits of one query head by one wave (flash_fwd_kernel.h:1217-1298 in unnormalised
-// form): out = sum_s w_s O_s / sum_s w_s L_s with w_s = 2^(M_s - max M).  Lane l owns channels 2l and
-// 2l+1.  Splits are taken N at a time (N = 32, or less when there are fewer splits): lane l holds the (M, L) pair of
-// split s0 + l % 32, the weights go back to all lanes as scalars.  The order of the additions is fixed: even
-// and odd splits of a block are summed separately (two dependent chains instead of one) and added at the end.
-// `split_stride` is in floats and, like the whole partial-output area, below 2^31 bytes (checked by the host).
+// Merge of the splits of one query head by one wave (flash_fwd_kernel.h:1217-1298 with normalised partials):
+// out = sum_s w_s O_s / sum_s w_s with w_s = 2^(M_s - max M) L_s and O_s the split's normalised output.
+// Lane l owns channels 2l and 2l+1.  Splits are taken N at a time (N = 32, or less when there are fewer splits):
+// lane l holds the (M, L) pair of split s0 + l % 32, the weights go back to all lanes as scalars.  The order of
+// the additions is fixed: even and odd splits of a block are summed separately (two dependent chains instead of
+// one) and added at the end.  On return O0, O1 are the weighted sums and L the sum of the weights (the head's
+// softmax denominator relative to M).  The partial-output area is below 2^31 bytes (checked by the host).
 template <int N>
-__device__ __forceinline__ void merge_splits_n(const float* o_part, const float* ml_part, int64_t hrow, uint32_t split_stride,
+__device__ __forceinline__ void merge_splits_n(const uint32_t* o_part, const float* ml_part, int64_t hrow,
                                                int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
-    const float* head_base = o_part + hrow * kHeadDim;
+    const uint32_t* head_base = o_part + hrow * nsplit * kPartialWords;
     const float* mlb = ml_part + hrow * nsplit * 2;
-    const uint32_t lane_bytes = lane * 8, ml_lane = (lane & 31) * 8;
+    const uint32_t lane_bytes = lane * 4, ml_lane = (lane & 31) * 8;
     const int sl = lane & 31;
     const float2 none = float2{-INFINITY, 0.0f};
-    float2 v[N];
+    uint32_t v[N];
     float2 ml = none;
     float lacc = 0.0f, Mu = 0.0f;
     float e0 = 0.0f, e1 = 0.0f, d0 = 0.0f, d1 = 0.0f;
     for (int s0 = 0; s0 < nsplit; s0 += 32) {
         if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
-        load_partials<N>(v, head_base, lane_bytes, split_stride, s0, nsplit);
+        load_partials<N>(v, head_base, lane_bytes, s0, nsplit);
         if (s0 == 0) {
             float mx = ml.x;
             for (int s = 32; s < nsplit; s += 32) {        // more than 32 splits: the other maxima
@@ -1094,15 +1118,15 @@ __device__ __forceinline__ void merge_splits_n(const float* o_part, const float*
             M = wave_max(mx);
             Mu = (M == -INFINITY) ? 0.0f : M;
         }
-        const float w = (s0 + sl < nsplit) ? __builtin_amdgcn_exp2f(ml.x - Mu) : 0.0f;
-        lacc = __builtin_fmaf(w, ml.y, lacc);
+        const float w = (s0 + sl < nsplit) ? __builtin_amdgcn_exp2f(ml.x - Mu) * ml.y : 0.0f;
+        lacc += w;
 #pragma unroll
         for (int k = 0; k < N; k += 2) {
             const float wa = lane_value(w, k), wb = lane_value(w, k + 1);
-            e0 = __builtin_fmaf(wa, v[k].x, e0);
-            e1 = __builtin_fmaf(wa, v[k].y, e1);
-            d0 = __builtin_fmaf(wb, v[k + 1].x, d0);
-            d1 = __builtin_fmaf(wb, v[k + 1].y, d1);
+            e0 = __builtin_fmaf(wa, partial_lo(v[k]), e0);
+            e1 = __builtin_fmaf(wa, partial_hi(v[k]), e1);
+            d0 = __builtin_fmaf(wb, partial_lo(v[k + 1]), d0);
+            d1 = __builtin_fmaf(wb, partial_hi(v[k + 1]), d1);
         }
     }
     O0 = e0 + d0;
@@ -1111,18 +1135,18 @@ __device__ __forceinline__ void merge_splits_n(const float* o_part, const float*
     const float lrow = row_sum16(lacc);
     L = lane_value(lrow, 0) + lane_value(lrow, 16);
 }
-__device__ __forceinline__ void merge_splits(const float* o_part, const float* ml_part, int64_t hrow, uint32_t split_stride,
+__device__ __forceinline__ void merge_splits(const uint32_t* o_part, const float* ml_part, int64_t hrow,
                                              int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
     // as many loads per lane as there are splits, rounded up to 4, 8, 16 or 32: every one of them is a round trip
     // of its own to the memory side (with 32 loads for 8 splits the 4K-token step took 0.5 us longer)
     if (nsplit <= 4) {
-        merge_splits_n<4>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<4>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
     } else if (nsplit <= 8) {
-        merge_splits_n<8>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<8>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
     } else if (nsplit <= 16) {
-        merge_splits_n<16>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<16>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
     } else {
-        merge_splits_n<32>(o_part, ml_part, hrow, split_stride, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<32>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
     }
 }
 
@@ -1455,25 +1479,23 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     uint16_t* out = P.out;
     int64_t out_sb = P.out_sb, out_sh = P.out_sh;
     float* lse_out = P.lse;
-    float* o_part = P.o_part;
+    uint32_t* o_part = P.o_part;
     float* ml_part = P.ml_part;
     int* tickets = P.tickets;
-    int n_h = P.h, n_b = P.b;
+    int n_h = P.h;
     if constexpr (APPEND) {      // as for the window: fetched late
         const kblock ob = karg_block<BLOCK_AT(o_part)>();       // o_part ... h
         out = BLOCK_PTR(uint16_t*, ob, o_part, out);
         out_sb = BLOCK_I64(ob, o_part, out_sb);
         out_sh = BLOCK_I64(ob, o_part, out_sh);
         lse_out = BLOCK_PTR(float*, ob, o_part, lse);
-        o_part = BLOCK_PTR(float*, ob, o_part, o_part);
+        o_part = BLOCK_PTR(uint32_t*, ob, o_part, o_part);
         ml_part = BLOCK_PTR(float*, ob, o_part, ml_part);
         tickets = BLOCK_PTR(int*, ob, o_part, tickets);
         n_h = BLOCK_I32(ob, o_part, h);
-        n_b = BLOCK_I32(ob, o_part, b);
     }
     const int hq = hk * g + wave;                                  // this wave's query head
     const int64_t hrow = static_cast<int64_t>(bi) * n_h + hq;      // its row in [b][h] tables
-    const int64_t hstride = static_cast<int64_t>(n_b) * n_h;       // rows per split in the workspace
     uint16_t* const out_row = out + bi * out_sb + hq * out_sh;
     if (wave < g) {
         // weights of the waves: lane (any row, w) takes wave w; the row reductions give every lane the
@@ -1496,7 +1518,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
         if (P.nsplit == 1) {
             write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
         } else {
-            st_dev2(&o_part[(split * hstride + hrow) * kHeadDim + 2 * lane], O0, O1);
+            st_dev1(&o_part[(hrow * P.nsplit + split) * kPartialWords + lane], pack_partial(O0, O1, L));
             if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M, L);
             wait_vm<0>();
             PROF(5);
@@ -1509,7 +1531,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
             if constexpr (APPEND) {
                 if (wave == 0) *s_last = last;
             } else if (last) {
-                merge_splits(o_part, ml_part, hrow, static_cast<uint32_t>(hstride) * kHeadDim, P.nsplit, lane, O0, O1, M, L);
+                merge_splits(o_part, ml_part, hrow, P.nsplit, lane, O0, O1, M, L);
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }
@@ -1524,7 +1546,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
             appends = *s_last != 0;
             if (appends) step_begin<NW>(bi, hk, step_len);
             if (wave < g && last) {
-                merge_splits(o_part, ml_part, hrow, static_cast<uint32_t>(hstride) * kHeadDim, P.nsplit, lane, O0, O1, M, L);
+                merge_splits(o_part, ml_part, hrow, P.nsplit, lane, O0, O1, M, L);
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }

@@ -9,6 +9,7 @@ namespace bitdecode {
 // same time: each sits in a 256-byte block of its own (counters that share a cache line cost several
 // microseconds per launch on a multi-die GPU, measured).
 constexpr int kTicketStride = 64;      // ints
+constexpr int kPartialWords = 64;      // 32-bit words of one split's partial output of one query head: 128 channels as fp16
 
 struct QpackParams {
     const uint16_t* k;
@@ -46,7 +47,7 @@ struct FwdParams {
     const int* seqlens;
     const int* reslens;
     int seqlen, reslen;
-    float* o_part;      // [split][b][h][128] partial outputs, relative to the split's own maximum
+    uint32_t* o_part;   // [b][h][split][64] partial outputs: normalised (O / sum), two fp16 channels per word
     float* ml_part;     // [b][h][split][2] maximum (base-2 units) and sum of each split
     int* tickets;       // [b][h] arrival counters, kTicketStride ints apart, zero between calls
     uint16_t* out;

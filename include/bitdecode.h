@@ -124,7 +124,7 @@ int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
  * results as bitdecode_fwd, except that `workspace` / `workspace_bytes` are ignored: partial outputs and
  * arrival counters live in an 8 MiB array inside the library's code object (one copy per GPU, held until the
- * process ends), and the call allocates nothing.  Limits: b * h <= 4096 and num_splits * b * h * 520 bytes
+ * process ends), and the call allocates nothing.  Limits: b * h <= 4096 and num_splits * b * h * 264 bytes
  * <= 7 MiB, otherwise BITDECODE_EWORKSPACE.  All calls on one GPU share that array: calls that overlap in
  * time on one GPU (two streams, two host threads) race; calls on one stream do not.  The first call on a
  * device looks up the array's address (hipGetSymbolAddress): make it outside any stream capture. */
@@ -167,7 +167,7 @@ size_t bitdecode_fwd_append_workspace_bytes(int32_t b, int32_t h, int32_t num_sp
 int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
                          int32_t num_cus, int32_t bits, int32_t group_size);
 
-/* Workspace the split path needs: arrival counters, fp32 partial outputs and LSEs
+/* Workspace the split path needs: arrival counters, partial outputs (normalised, fp16) and fp32 (max, sum) pairs
  * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,
  * csrc/bit_decode/decode_api.cpp:292-295). */
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits);

@@ -267,8 +267,8 @@ def test_split_choice_and_workspace_size():
     assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256, 4, 128) == 6
     assert lib.bitdecode_num_splits(1, 1, 1024, 0, 256, 3, 128) == -1
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
-    # one 256-byte counter block per query head + fp32 partial outputs and (max, sum) pairs per split
-    assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 32 * 256 + 32 * 32 * 130 * 4
+    # one 256-byte counter block per query head + fp16 partial outputs and fp32 (max, sum) pairs per split
+    assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 32 * 256 + 32 * 32 * 66 * 4
 
 
 def test_python_entry_points_validate_before_touching_the_gpu():

@@ -64,8 +64,9 @@ def test_static_scratch_entry_matches_the_workspace_entry(device):
 
     # beyond the built-in scratch: a clear error, nothing launched
     L = _lib.lib()
+    wide = _plan(device, 34, 2, 32, 8, 8192, 128, 4, 128, 0)
     a = _lib.FwdArgs()
-    ctypes.memmove(ctypes.byref(a), ctypes.byref(big.args), ctypes.sizeof(a))
-    a.num_splits = 512                                             # 512 x 32 rows x 520 B = 8.5 MB > 7 MiB
+    ctypes.memmove(ctypes.byref(a), ctypes.byref(wide.args), ctypes.sizeof(a))
+    a.num_splits = 512                                             # 512 x 64 rows x 264 B = 8.65 MB > 7 MiB
     rc = L.bitdecode_fwd_static(ctypes.byref(a), torch.cuda.current_stream(device).cuda_stream)
     assert rc == 3 and b"built-in scratch" in L.bitdecode_last_error()
