@@ -70,7 +70,7 @@ class FwdAppendArgs(ctypes.Structure):
 
 
 EXPORTS = ("bitdecode_abi_version", "bitdecode_last_error", "bitdecode_num_splits",
-           "bitdecode_fwd_workspace_bytes", "bitdecode_qpack", "bitdecode_fwd",
+           "bitdecode_fwd_workspace_bytes", "bitdecode_num_splits_for", "bitdecode_qpack", "bitdecode_fwd",
            "bitdecode_fwd_append", "bitdecode_fwd_append_workspace_bytes", "bitdecode_read_probe", "bitdecode_fwd_static")
 
 _lib = None
@@ -98,6 +98,8 @@ def lib():
         L.bitdecode_last_error.restype = ctypes.c_char_p
         L.bitdecode_num_splits.restype = ctypes.c_int
         L.bitdecode_num_splits.argtypes = [_i32] * 7
+        L.bitdecode_num_splits_for.restype = ctypes.c_int
+        L.bitdecode_num_splits_for.argtypes = [_i32] * 8
         L.bitdecode_fwd_workspace_bytes.restype = ctypes.c_size_t
         L.bitdecode_fwd_workspace_bytes.argtypes = [_i32] * 3
         L.bitdecode_qpack.restype = ctypes.c_int

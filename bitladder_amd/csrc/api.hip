@@ -86,6 +86,33 @@ int choose_splits(int b, int hk, int max_seqlen_k, int max_res_len, int num_cus,
     return std::max(1, n);
 }
 
+// The 4-bit kernels also exist with 8 waves per workgroup (decode.hip: launch_fwd_tt), used whenever the packed
+// prefix is the bulk of the work.  With per-sequence lengths on the device the workgroups of the longest
+// sequences can be left streaming alone at the end, where 16 waves keep more bytes in flight per compute
+// unit: then only up to 32 units per workgroup (measured on a batch of 16 sequences of 1.9K-8K tokens: 26.2
+// against 26.6 us; equal-length batches of every size measured gain 1-7 % from the 8 waves).
+bool use_few_waves(int bits, int gs, int max_s, int max_r, int nsplit, bool device_lengths) {
+    const int packed_units = max_s / bitdecode::unit_tokens(bits);
+    const int units_per_wg = (packed_units + nsplit - 1) / nsplit;
+    return bitdecode::few_waves_variant(bits, gs) && units_per_wg >= 1 && max_r <= 512 &&
+           (!device_lengths || units_per_wg <= 32);
+}
+
+// Split count for a call; `ragged` = per-sequence lengths come from the device (the host only has their bound).
+// Two workgroups of the 8-wave kernels fit a compute unit (78 KB of LDS and 125 registers each).  A batch of
+// unequal sequences is better served by twice as many workgroups of half the size: the two that share a unit
+// add up, and the kernel orders the sequences so that the longest shares with the shortest (decode.hip:
+// sequence_of_position).  16 sequences of 1.9K-8K tokens: 62 units on the busiest unit with one workgroup
+// per unit, 49.5 with two.
+int choose_splits_for(int b, int hk, int max_s, int max_r, int num_cus, int bits, int gs, bool ragged) {
+    const int n1 = choose_splits(b, hk, max_s, max_r, num_cus, bits, gs);
+    if (!ragged || b < 2) return n1;
+    const int n2 = choose_splits(b, hk, max_s, max_r, 2 * num_cus, bits, gs);
+    if (n2 > n1 && static_cast<int64_t>(n2) * b * hk <= 2 * num_cus && use_few_waves(bits, gs, max_s, max_r, n2, true))
+        return n2;
+    return n1;
+}
+
 }  // namespace
 
 extern "C" {
@@ -99,6 +126,13 @@ int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t m
     if (num_cus <= 0) num_cus = query_cus();
     if (check_quant(bits, group_size, BITDECODE_FP16, bitdecode::kHeadDim)) return -1;
     return choose_splits(b, h_k, max_seqlen_k, max_res_len, num_cus, bits, group_size);
+}
+
+int bitdecode_num_splits_for(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len, int32_t num_cus,
+                             int32_t bits, int32_t group_size, int32_t per_sequence_lengths) {
+    if (num_cus <= 0) num_cus = query_cus();
+    if (check_quant(bits, group_size, BITDECODE_FP16, bitdecode::kHeadDim)) return -1;
+    return choose_splits_for(b, h_k, max_seqlen_k, max_res_len, num_cus, bits, group_size, per_sequence_lengths != 0);
 }
 
 // [tickets: one 256-byte block per (batch, query head)][o_part][ml_part]
@@ -249,7 +283,9 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     int nsplit = a->num_splits;
     if (nsplit < 0) return fail(BITDECODE_EINVAL, "num_splits %d is negative", nsplit);
     if (nsplit > 512) return fail(BITDECODE_EINVAL, "num_splits %d is above the limit of 512", nsplit);
-    if (nsplit == 0) nsplit = choose_splits(a->b, a->h_k, max_s, max_r, query_cus(), a->bits, a->group_size);
+    const int cus = query_cus();
+    if (nsplit == 0)
+        nsplit = choose_splits_for(a->b, a->h_k, max_s, max_r, cus, a->bits, a->group_size, a->seqlens_k && !step);
     if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords * sizeof(uint32_t) >= (size_t(1) << 31))
         return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d heads: partial outputs of 2 GiB or more", nsplit, a->b, a->h);
     // the kernel divides workgroup ids and unit counts by the split count and the head count with a
@@ -303,18 +339,11 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     P.scale_log2 = fabsf(a->softmax_scale) * 1.4426950408889634f;   // decode_api.cpp:128-142
     P.neg_scale = a->softmax_scale < 0.0f;
     P.xcd_remap = (a->b * a->h_k) % 8 == 0 && nsplit > 1;
-    {
-        // The 4-bit kernels run with 8 waves per workgroup (decode.hip: launch_fwd_tt) whenever the packed prefix
-        // is the bulk of the work.  With per-sequence lengths on the device the workgroups of the longest sequences
-        // can be left streaming alone at the end, where 16 waves keep more bytes in flight per compute unit: then
-        // only up to 32 units per workgroup (measured on a batch of 16 sequences of 1.9K-8K tokens: 26.2 against
-        // 26.6 us; equal-length batches of every size measured gain 1-7 % from the 8 waves).
-        const int packed_units = max_s / bitdecode::unit_tokens(a->bits);
-        const int units_per_wg = (packed_units + nsplit - 1) / nsplit;
-        const bool device_lengths = a->seqlens_k != nullptr || step != nullptr;
-        P.few_waves = bitdecode::few_waves_variant(a->bits, a->group_size) && units_per_wg >= 1 && max_r <= 512 &&
-                      (!device_lengths || units_per_wg <= 32);
-    }
+    P.few_waves = use_few_waves(a->bits, a->group_size, max_s, max_r, nsplit, a->seqlens_k != nullptr || step != nullptr);
+    // more than one workgroup per compute unit and lengths that differ: the kernel deals the sequences out so
+    // that long ones share a unit with short ones (a pure permutation of the batch index, from the lengths
+    // on the device; not in the step with append, whose launch itself advances the lengths)
+    P.seq_perm = a->seqlens_k && !step && a->b >= 2 && a->b <= 64 && static_cast<int64_t>(nsplit) * a->b * a->h_k > cus;
     P.nsplit_magic = division_magic(static_cast<uint32_t>(nsplit));
     P.hk_magic = division_magic(static_cast<uint32_t>(a->h_k));
     P.block_table = a->block_table; P.bt_stride = a->block_table_stride;

@@ -1262,6 +1262,28 @@ __device__ __forceinline__ void step_end(uint8_t* lds, int bi, int hk, int t) {
     }
 }
 
+// With two workgroups per compute unit (the 8-wave kernels) and sequences of different lengths, the time of
+// a launch is that of the unit whose two workgroups add up to the most.  The dispatcher fills the units
+// round-robin, so the workgroups at batch positions p and p + b/2 share a unit: position p takes the p-th
+// longest sequence and position ceil(b/2) + k the k-th shortest, which pairs the longest with the shortest.
+// A permutation of the batch index computed by every wave from the device-side lengths (lane j holds sequence
+// j; equal lengths are ordered by index), so every workgroup arrives at the same one; the lengths are not
+// written during the launch.  Nothing else depends on it: results are indexed by the sequence.
+__device__ __forceinline__ int sequence_of_position(const FwdParams& P, int p, int lane) {
+    const int n = P.b;      // at most 64 (host)
+    int len = -1;
+    if (lane < n) len = min(max(P.seqlens[lane], 0), P.capacity);
+    int rank = 0;           // sequences that come before this lane's in descending order of length
+    for (int j = 0; j < n; ++j) {
+        const int lj = __builtin_amdgcn_readlane(len, j);
+        rank += (lj > len || (lj == len && j < lane)) ? 1 : 0;
+    }
+    const int half = (n + 1) >> 1;
+    const int pos = rank < half ? rank : half + (n - 1 - rank);
+    const unsigned long long hit = __ballot(lane < n && pos == p);
+    return __builtin_amdgcn_readfirstlane(static_cast<int>(__builtin_ctzll(hit)));
+}
+
 // ---------------------------------------------------------------------------------------------
 // split-KV kernel: 1-D grid of num_splits * h_k * b workgroups of UnitCfg::NW waves.
 // Split s of a (batch, kv-head) owns packed units [s*ups, (s+1)*ups) dealt round-robin to its
@@ -1315,6 +1337,9 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     }
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: unit addresses stay in SGPRs
+    if constexpr (!APPEND) {
+        if (P.seq_perm) bi = sequence_of_position(P, bi, lane);
+    }
     const int col = lane & 15, kg = lane >> 4;
     const int head = col & 7;          // query head inside the GQA group
     const bool lo_part = col >= 8;     // columns 8-15 carry the lo halves of the split products

@@ -77,6 +77,7 @@ struct FwdParams {
     // (a runtime integer division costs the prologue of every workgroup some 100 cycles, and there were five)
     uint32_t nsplit_magic, hk_magic;
     int few_waves;              // run the 8-wave variant of the kernel (layout.h: few_waves_variant)
+    int seq_perm;               // workgroups take their sequence by rank of length (decode.hip: sequence_of_position)
 };
 
 inline uint32_t division_magic(uint32_t d) { return d <= 1 ? 0u : static_cast<uint32_t>(((1ull << 32) + d - 1) / d); }

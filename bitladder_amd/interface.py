@@ -141,14 +141,15 @@ def _stream_workspace(device, kind: str, b: int, h: int, ns: int, nbytes: int) -
 _SPLIT_PLANS: "dict[tuple, tuple]" = {}
 
 
-def _split_plan(dev_index, b, h, h_k, max_seqlen, max_res, new_tokens, bits, gs, num_splits):
+def _split_plan(dev_index, b, h, h_k, max_seqlen, max_res, ragged, bits, gs, num_splits):
     """(split count, workspace bytes) of a decode call on the current device; both are pure functions of
-    these arguments (and of the device's compute-unit count), so the two library calls are made once."""
-    key = (dev_index, b, h, h_k, max_seqlen, max_res, new_tokens, bits, gs, num_splits)
+    these arguments (and of the device's compute-unit count), so the two library calls are made once.
+    `ragged`: the call takes per-sequence packed lengths from the device."""
+    key = (dev_index, b, h, h_k, max_seqlen, max_res, ragged, bits, gs, num_splits)
     hit = _SPLIT_PLANS.get(key)
     if hit is None:
         L = _lib.lib()
-        ns = num_splits or L.bitdecode_num_splits(b, h_k, max_seqlen, max_res, new_tokens, bits, gs)
+        ns = num_splits or L.bitdecode_num_splits_for(b, h_k, max_seqlen, max_res, 0, bits, gs, int(ragged))
         hit = (ns, L.bitdecode_fwd_workspace_bytes(b, h, ns))
         if len(_SPLIT_PLANS) >= 4096:
             _SPLIT_PLANS.clear()
@@ -423,8 +424,8 @@ def plan_fwd_kvcache_int(q: torch.Tensor,
     a.quant_mode = mode
     a.softmax_scale = float(softmax_scale)
     with _on_device(device):
-        ns, nbytes = _split_plan(device.index, b, h, h_k, a.max_seqlen_k, a.max_res_len, 0, num_bits, group_size,
-                                 int(num_splits))
+        ns, nbytes = _split_plan(device.index, b, h, h_k, a.max_seqlen_k, a.max_res_len, seqlens_k is not None,
+                                 num_bits, group_size, int(num_splits))
         a.num_splits = ns
         if nbytes:
             # zero-filled: the arrival counters at its head must be 0 before the first call

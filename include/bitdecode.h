@@ -167,6 +167,13 @@ size_t bitdecode_fwd_append_workspace_bytes(int32_t b, int32_t h, int32_t num_sp
 int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
                          int32_t num_cus, int32_t bits, int32_t group_size);
 
+/* The same for a call that takes per-sequence lengths from the device (bitdecode_fwd_args.seqlens_k) when
+ * per_sequence_lengths != 0: a batch of unequal sequences gets up to two workgroups per compute unit, dealt
+ * out so that long sequences share a unit with short ones.  This is the count bitdecode_fwd chooses itself
+ * with num_splits = 0.  No counterpart in the reference, whose heuristic only sees the longest sequence. */
+int bitdecode_num_splits_for(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
+                             int32_t num_cus, int32_t bits, int32_t group_size, int32_t per_sequence_lengths);
+
 /* Workspace the split path needs: arrival counters, partial outputs (normalised, fp16) and fp32 (max, sum) pairs
  * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,
  * csrc/bit_decode/decode_api.cpp:292-295). */

@@ -262,6 +262,36 @@ def test_decode_random_shapes(device, seed):
         assert torch.equal(again, out)
 
 
+@pytest.mark.parametrize("b,lengths", [(5, [1024, 0, 1024, 384, 2048]), (16, None), (2, [128, 2048]), (64, None)])
+def test_sequences_dealt_out_by_length_give_the_same_bits(device, b, lengths):
+    """More workgroups than compute units and per-sequence lengths on the device: the kernel permutes the batch
+    index by rank of length (ties by index; odd batch sizes; empty sequences).  The permutation must not change a
+    bit: every sequence's output equals that of a call over that sequence alone with the same split count, and
+    matches the oracle."""
+    from bitladder_amd import fwd_kvcache_int
+    h_k, g, S, R, bits, gs = 8, 2, 2048, 40, 4, 128
+    if b == 64:
+        h_k, g = 2, 4
+    h = h_k * g
+    rng = np.random.default_rng(b)
+    seqlens = np.asarray(lengths if lengths is not None else 128 * rng.integers(0, S // 128 + 1, b), dtype=np.int32)
+    ns = max(2, -(-300 // (b * h_k)))                     # b * h_k * ns > 256 compute units
+    q, k, v = O.make_inputs(b, h, h_k, S, R, seed=77 + b)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    qd = H.to_dev(q, "fp16", device)
+    kr, vr = H.to_dev(k[:, S:], "fp16", device), H.to_dev(v[:, S:], "fp16", device)
+    out = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, seqlens_k=torch.from_numpy(seqlens).to(device),
+                          max_seqlen_k=S, k_residual=kr, v_residual=vr, num_splits=ns)
+    for i in range(b):      # alone, with a host-side length: a grid without the permutation
+        alone = fwd_kvcache_int(qd[i:i + 1], *(t[i:i + 1] for t in cache), None, SCALE, "k-channel", gs, bits,
+                                seqlen_k=int(seqlens[i]), k_residual=kr[i:i + 1], v_residual=vr[i:i + 1], num_splits=ns)
+        assert torch.equal(out[i:i + 1], alone), (i, int(seqlens[i]))
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, _ = O.attend_ref(q, k_hat, v_hat, SCALE, k[:, S:], v[:, S:], seqlens_k=seqlens)
+    assert np.abs(out.float().cpu().numpy() - want).max() < ATOL
+
+
 @pytest.mark.parametrize("bits", [2, 4])
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 def test_qpack_ranges_from_subnormal_to_max(device, bits, dtype):

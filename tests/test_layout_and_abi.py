@@ -266,6 +266,14 @@ def test_split_choice_and_workspace_size():
     # 48 units, at least one unit for every second of the 16 waves -> 6 splits
     assert lib.bitdecode_num_splits(1, 1, 128 * 24, 0, 256, 4, 128) == 6
     assert lib.bitdecode_num_splits(1, 1, 1024, 0, 256, 3, 128) == -1
+    # per-sequence lengths on the device: a batch of 16 gets two workgroups of the 8-wave kernel per compute unit
+    assert lib.bitdecode_num_splits(16, 8, 8192, 256, 256, 4, 128) == 2
+    assert lib.bitdecode_num_splits_for(16, 8, 8192, 256, 256, 4, 128, 0) == 2
+    assert lib.bitdecode_num_splits_for(16, 8, 8192, 256, 256, 4, 128, 1) == 4
+    # ... not the 2-bit kernels (16 waves, one workgroup per unit), not one sequence, not workgroups of more than 32 units
+    assert lib.bitdecode_num_splits_for(16, 8, 8192, 256, 256, 2, 128, 1) == 2
+    assert lib.bitdecode_num_splits_for(1, 8, 32768, 128, 256, 4, 128, 1) == 32
+    assert lib.bitdecode_num_splits_for(16, 8, 65536, 128, 256, 4, 128, 1) == 2
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
     # one 256-byte counter block per query head + fp16 partial outputs and fp32 (max, sum) pairs per split
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 32 * 256 + 32 * 32 * 66 * 4
