@@ -31,7 +31,7 @@ MEASURED_TRAFFIC_BYTES = {
     "llama3-8b-gqa-32k-4bit-g128": int(17965.51 * 2048 + 329.00 * 1024),
     "llama2-7b-mha-4k-4bit-g128": int(9886.52 * 2048 + 89.00 * 1024),
     "llama3-8b-gqa-128k-2bit-g64": int(41569.52 * 2048 + 329.00 * 1024),
-    "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": int(55899.39 * 2048 + 464.00 * 1024),
+    "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": int(56131.44 * 2048 + 784.00 * 1024),
     "llama3-70b-gqa-64k-2bit-g128-b8": int(150022.50 * 2048 + 784.00 * 1024),
 }
 

@@ -103,10 +103,12 @@ bool use_few_waves(int bits, int gs, int max_s, int max_r, int nsplit, bool devi
 // unequal sequences is better served by twice as many workgroups of half the size: the two that share a unit
 // add up, and the kernel orders the sequences so that the longest shares with the shortest (decode.hip:
 // sequence_of_position).  16 sequences of 1.9K-8K tokens: 62 units on the busiest unit with one workgroup
-// per unit, 49.5 with two.
+// per unit, 49.5 with two.  Only for batches that fill the machine with one or two splits: the host cannot tell a
+// ragged batch from an equal one, and equal sequences lose by the doubling what the extra splits cost
+// (32 x 8 heads: nothing; 16 x 8: 1.5 %; 8 x 8 and 4 x 8, where 4 and 8 splits would become 8 and 16: 9-12 %).
 int choose_splits_for(int b, int hk, int max_s, int max_r, int num_cus, int bits, int gs, bool ragged) {
     const int n1 = choose_splits(b, hk, max_s, max_r, num_cus, bits, gs);
-    if (!ragged || b < 2) return n1;
+    if (!ragged || b < 2 || n1 > 2) return n1;
     const int n2 = choose_splits(b, hk, max_s, max_r, 2 * num_cus, bits, gs);
     if (n2 > n1 && static_cast<int64_t>(n2) * b * hk <= 2 * num_cus && use_few_waves(bits, gs, max_s, max_r, n2, true))
         return n2;

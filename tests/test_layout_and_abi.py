@@ -274,6 +274,8 @@ def test_split_choice_and_workspace_size():
     assert lib.bitdecode_num_splits_for(16, 8, 8192, 256, 256, 2, 128, 1) == 2
     assert lib.bitdecode_num_splits_for(1, 8, 32768, 128, 256, 4, 128, 1) == 32
     assert lib.bitdecode_num_splits_for(16, 8, 65536, 128, 256, 4, 128, 1) == 2
+    # ... and not batches that need more than two splits to fill the machine anyway
+    assert lib.bitdecode_num_splits_for(8, 8, 8192, 128, 256, 4, 128, 1) == lib.bitdecode_num_splits(8, 8, 8192, 128, 256, 4, 128) == 4
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
     # one 256-byte counter block per query head + fp16 partial outputs and fp32 (max, sum) pairs per split
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 32 * 256 + 32 * 32 * 66 * 4
