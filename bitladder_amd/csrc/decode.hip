@@ -34,7 +34,7 @@
 //    shared by the four lanes of a head through two lane-half swaps, accumulators rescaled only
 //    when some head's max actually moved.
 //  * The waves of a workgroup merge through LDS, one wave per query head; splits merge in the
-//    same launch: that wave publishes the head's unnormalised (O, max, sum), draws a ticket from
+//    same launch: that wave publishes the head's (O / sum in fp16, max, sum), draws a ticket from
 //    the head's counter, and the wave that draws the last one combines all splits of the head.
 #include <hip/hip_runtime.h>
 #include <stddef.h>
@@ -1288,8 +1288,8 @@ __device__ __forceinline__ int sequence_of_position(const FwdParams& P, int p, i
 // split-KV kernel: 1-D grid of num_splits * h_k * b workgroups of UnitCfg::NW waves.
 // Split s of a (batch, kv-head) owns packed units [s*ups, (s+1)*ups) dealt round-robin to its
 // waves; the 16-token tiles of the fp16 window are dealt round-robin over ALL waves of the head.
-// With more than one split each workgroup writes its unnormalised (O, max, sum) and takes a ticket;
-// the workgroup that draws the last ticket of its (batch, kv-head) merges all partials
+// With more than one split each head's wave writes its (O / sum in fp16, max, sum) and takes a ticket of the head;
+// the wave that draws the last ticket merges all partials of the head
 // (flash_fwd_kernel.h:1217-1298 formula) and resets the ticket.
 //
 // Dynamic LDS: [NW wave regions of UnitCfg::REGION bytes][q: 8 head rows + a zero row, 272 B apart]
