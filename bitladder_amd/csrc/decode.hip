@@ -1281,7 +1281,8 @@ __device__ __forceinline__ int sequence_of_position(const FwdParams& P, int p, i
     const int half = (n + 1) >> 1;
     const int pos = rank < half ? rank : half + (n - 1 - rank);
     const unsigned long long hit = __ballot(lane < n && pos == p);
-    return __builtin_amdgcn_readfirstlane(static_cast<int>(__builtin_ctzll(hit)));
+    // (pos is a permutation of 0 .. n-1, so exactly one lane answers; p itself if that were ever not so)
+    return __builtin_amdgcn_readfirstlane(hit ? static_cast<int>(__builtin_ctzll(hit)) : p);
 }
 
 // ---------------------------------------------------------------------------------------------
