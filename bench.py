@@ -56,6 +56,10 @@ WORKLOADS = {
     "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": (16, 32, 8, 8192, 256, 4, 128, torch.float16),
 }
 RAGGED = {"llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": (1024, 8192)}
+DEFAULT_WORKLOAD = "llama3-8b-gqa-32k-4bit-g128"
+# the other four BASELINE shapes, timed compactly by the default run ("other_configs")
+OTHER_CONFIGS = ("llama2-7b-mha-4k-4bit-g128", "llama3-8b-gqa-128k-2bit-g64",
+                 "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128", "llama3-70b-gqa-64k-2bit-g128-b8")
 
 
 def ragged_lengths(name, b):
@@ -93,6 +97,90 @@ def alloc_cache(b, S, h_k, bits, gs, dev):
             torch.zeros((b, S // gs, h_k, 128), dtype=torch.float32, device=dev),
             torch.zeros((b, S, h_k, 128 // pn), dtype=torch.uint16, device=dev),
             torch.zeros((b, 128 // gs, h_k, S), dtype=torch.float32, device=dev))
+
+
+def workload_bytes(name):
+    """(algorithmic bytes per step, of which packed stream, packed lengths, window lengths) of a workload; the
+    lengths are None unless the workload is ragged."""
+    b, h, h_k, S, R, bits, gs, _ = WORKLOADS[name]
+    if name in RAGGED:
+        packed_len, win_len = ragged_lengths(name, b)
+        per_tok = h_k * 128 * 2
+        packed_bytes = int(packed_len.sum().item() * per_tok * (bits / 8 + 4 / gs))
+        total_bytes = packed_bytes + int(win_len.sum().item()) * per_tok * 2 + 2 * b * h * 128 * 2
+        return total_bytes, packed_bytes, packed_len, win_len
+    total_bytes, packed_bytes = algorithmic_bytes(b, h, h_k, S, R, bits, gs)
+    return total_bytes, packed_bytes, None, None
+
+
+def make_inputs_gpu(b, h, h_k, n_tokens, seed, dtype, dev):
+    """The same distribution generated on the GPU (for the workloads no CPU checker looks at)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q = torch.randn((b, 1, h, 128), generator=g, device=dev).to(dtype)
+    k = torch.randn((b, n_tokens, h_k, 128), generator=g, device=dev, dtype=torch.float16).to(dtype)
+    v = torch.randn((b, n_tokens, h_k, 128), generator=g, device=dev, dtype=torch.float16).to(dtype)
+    for hk in range(h_k):
+        ch = torch.randperm(128, generator=g, device=dev)[:3]
+        k[:, :, hk, ch] *= 10.0
+    return q, k, v
+
+
+def build_workload(name, num_splits=0, no_rotate=False, want_sources=False, cpu_inputs=True, max_bufs=16):
+    """Packed caches, windows and decode plans of a workload: enough distinct caches that consecutive steps
+    cannot be served from the 256 MB Infinity Cache.  With `cpu_inputs` every cache gets its own CPU-seeded
+    tensors (a CPU checker sees the same bits); otherwise two GPU-generated sources are packed in turn."""
+    from bitladder_amd import kvcache_pack_int, plan_fwd_kvcache_int
+    dev = torch.device("cuda:0")
+    b, h, h_k, S, R, bits, gs, dtype = WORKLOADS[name]
+    scale = 1.0 / math.sqrt(128)
+    ragged = name in RAGGED
+    total_bytes, packed_bytes, packed_len, win_len = workload_bytes(name)
+    if ragged:
+        packed_dev, win_dev = packed_len.to(dev), win_len.to(dev)
+    nbuf = 1 if no_rotate else max(2, math.ceil(320e6 / total_bytes))
+    nbuf = min(nbuf, max_bufs)
+    plans, keep, srcs = [], [], []
+    first = None
+    gpu_src = []
+    for i in range(nbuf):
+        if cpu_inputs:
+            q, k, v = make_inputs(b, h, h_k, S + R, seed=i, dtype=dtype)
+            if i == 0:
+                first = (q, k, v)
+            qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+        else:
+            if i < 2:
+                gpu_src.append(make_inputs_gpu(b, h, h_k, S + R, i, dtype, dev))
+            qd, kd, vd = gpu_src[i % 2]
+        cache = alloc_cache(b, S, h_k, bits, gs, dev)
+        kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S,
+                         "k-channel", gs, bits)
+        if ragged:
+            # window of sequence j: its tokens behind the packed prefix
+            kres = torch.zeros((b, R, h_k, 128), dtype=dtype, device=dev)
+            vres = torch.zeros_like(kres)
+            for j in range(b):
+                p0, r0 = int(packed_len[j]), int(win_len[j])
+                kres[j, :r0], vres[j, :r0] = kd[j, p0:p0 + r0], vd[j, p0:p0 + r0]
+            plan = plan_fwd_kvcache_int(qd, *cache, None, scale, "k-channel", gs, bits,
+                                        seqlens_k=packed_dev, max_seqlen_k=int(packed_len.max()),
+                                        k_residual=kres, v_residual=vres, residual_len=win_dev,
+                                        max_residual_len=int(win_len.max()), num_splits=num_splits)
+        else:
+            kres, vres = kd[:, S:].contiguous(), vd[:, S:].contiguous()
+            plan = plan_fwd_kvcache_int(qd, *cache, None, scale, "k-channel", gs, bits,
+                                        k_residual=kres, v_residual=vres, num_splits=num_splits)
+        plans.append(plan)
+        keep.append((cache, kres, vres))
+        if want_sources and (i < 2 or sum(a.numel() + b_.numel() for a, b_ in srcs) * 2 < 640e6):
+            # fp16 sources for the quantize-pack leg: at least two, and enough of them (more than twice the
+            # 256 MB Infinity Cache in total) that no pack call finds its input cached
+            srcs.append((kd, vd))
+        del kd, vd
+    del gpu_src
+    torch.cuda.synchronize(dev)
+    return {"nbuf": nbuf, "plans": plans, "keep": keep, "srcs": srcs, "first_inputs": first or (None, None, None),
+            "total_bytes": total_bytes, "packed_bytes": packed_bytes}
 
 
 MIN_GRAPH_NODES = 200      # steps captured into one graph (a multiple of --steps): keeps the gaps between graph launches rare
@@ -175,6 +263,110 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True,
     return res
 
 
+# Read probe (libbitdecode_probe.so, built next to the library; a measurement aid of this file only): kernels that
+# read a buffer and do nothing else.  A configuration is (workgroups, threads, mode, depth, nt, pattern); see
+# bitladder_amd/csrc/probe.hip.
+PROBE_DEFAULT = [   # the configurations the sweep (--probe-sweep) found fastest at one size or another
+    (256, 1024, 0, 8, 1, 0),
+    (512, 512, 0, 8, 1, 0),
+    (1024, 256, 0, 8, 1, 0),
+    (256, 1024, 1, 4, 1, 1),
+    (512, 512, 0, 16, 1, 0),
+]
+_probe_lib = None
+
+
+def probe_lib():
+    global _probe_lib
+    if _probe_lib is None:
+        import ctypes
+        path = os.path.join(ROOT, "bitladder_amd", "libbitdecode_probe.so")
+        if not os.path.exists(path):
+            raise ImportError(f"{path} is missing: build it with `python -m bitladder_amd.build`")
+        L = ctypes.CDLL(path)
+        L.bitprobe_read.restype = ctypes.c_int
+        L.bitprobe_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t] + [ctypes.c_int] * 6 + [ctypes.c_void_p]
+        _probe_lib = L
+    return _probe_lib
+
+
+def probe_name(cfg):
+    g, t, mode, depth, nt, pat = cfg
+    return "%dx%d %s depth %d%s %s" % (g, t, "lds-dma" if mode else "regs", depth, " nt" if nt else "",
+                                     "wg-contiguous" if pat else "round-robin")
+
+
+def time_probe(nbytes, cfg, steps, warmup, use_graph, bufs, steady=True):
+    """us per launch of one read-probe configuration over `nbytes` (rotated buffers); None if it is not built."""
+    L = probe_lib()
+    dev = torch.device("cuda:0")
+    g, t, mode, depth, nt, pat = cfg
+
+    def probe(i):
+        buf = bufs[i % len(bufs)]
+        if L.bitprobe_read(buf.data_ptr(), nbytes, g, t, mode, depth, nt, pat, torch.cuda.current_stream(dev).cuda_stream):
+            raise RuntimeError("probe configuration not available")
+    try:
+        probe(0)
+    except RuntimeError:
+        return None
+    return time_steps(probe, steps, warmup, use_graph, steady=steady)["event_us"]
+
+
+def best_probe(nbytes, steps, warmup, use_graph, nbuf, configs=None):
+    """(us, configuration name, all timings) of the fastest read-probe configuration over `nbytes`."""
+    dev = torch.device("cuda:0")
+    nbytes = (nbytes + 4095) // 4096 * 4096
+    bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
+    seen = {}
+    for cfg in configs or PROBE_DEFAULT:
+        us = time_probe(nbytes, cfg, steps, warmup, use_graph, bufs)
+        if us is not None:
+            seen[probe_name(cfg)] = round(us, 3)
+    name = min(seen, key=seen.get)
+    return seen[name], name, seen, nbytes
+
+
+def probe_sweep(args):
+    """Table of the read probe over launch shapes and sizes (markdown on stdout)."""
+    dev = torch.device("cuda:0")
+    sizes = {"20 MB (4K MHA 4-bit)": workload_bytes("llama2-7b-mha-4k-4bit-g128")[0],
+             "36 MB (32K GQA 4-bit)": workload_bytes("llama3-8b-gqa-32k-4bit-g128")[0],
+             "84 MB (128K GQA 2-bit)": workload_bytes("llama3-8b-gqa-128k-2bit-g64")[0],
+             "306 MB (b8 64K 2-bit)": workload_bytes("llama3-70b-gqa-64k-2bit-g128-b8")[0]}
+    configs = []
+    for g in (256, 512, 1024):
+        for t in (256, 512, 1024):
+            for nt in (1, 0):
+                for pat in (0, 1):
+                    for depth in (4, 8, 16):
+                        configs.append((g, t, 0, depth, nt, pat))
+                    for depth in (4, 8):
+                        if (t // 64) * depth <= 128:
+                            configs.append((g, t, 1, depth, nt, pat))
+    rows = {probe_name(c): {} for c in configs}
+    for label, nbytes in sizes.items():
+        nbytes = (nbytes + 4095) // 4096 * 4096
+        nbuf = max(2, min(16, math.ceil(320e6 / nbytes)))
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
+        for c in configs:
+            us = time_probe(nbytes, c, 200, 5, True, bufs)
+            rows[probe_name(c)][label] = us
+            print("[sweep] %s | %s | %s" % (label, probe_name(c), "n/a" if us is None else "%.2f" % us),
+                  file=sys.stderr, flush=True)
+        del bufs
+    print("| configuration | " + " | ".join(sizes) + " |")
+    print("|---|" + "---|" * len(sizes))
+    for name, r in rows.items():
+        print("| %s | " % name + " | ".join("n/a" if r[k] is None else "%.2f" % r[k] for k in sizes) + " |")
+    print()
+    for label, nbytes in sizes.items():
+        ok = {n: r[label] for n, r in rows.items() if r[label] is not None}
+        n = min(ok, key=ok.get)
+        print("best at %s: %s, %.2f us = %.0f GB/s" % (label, n, ok[n], nbytes / ok[n] / 1e3))
+    return 0
+
+
 def cpu_baseline(q, k, v, S, R, bits, gs, scale, budget_s=20.0):
     """Reference semantics on the host cores: the torch oracle (dequantize the packed cache to
     fp32, fp32 softmax attention over [packed || residual]) timed on the same inputs."""
@@ -198,7 +390,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="llama3-8b-gqa-32k-4bit-g128", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of one HIP graph")
     ap.add_argument("--no-rotate", action="store_true", help="reuse one KV cache (stays in the 256 MB Infinity Cache)")
@@ -208,6 +400,9 @@ def main():
     ap.add_argument("--no-step", action="store_true", help="skip the decode-step-with-append leg")
     ap.add_argument("--no-dropin", action="store_true", help="skip the eager drop-in call leg")
     ap.add_argument("--no-probe", action="store_true", help="skip the read-probe leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the compact timing of the other BASELINE shapes")
+    ap.add_argument("--probe-sweep", action="store_true",
+                    help="only sweep the read probe over launch shapes and sizes and print the table")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three plain 256 MiB device copies (a kernel of known traffic, used to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -224,54 +419,19 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.probe_sweep:
+        return probe_sweep(args)
     b, h, h_k, S, R, bits, gs, dtype = WORKLOADS[args.workload]
     scale = 1.0 / math.sqrt(128)
     ragged = args.workload in RAGGED
+    total_bytes, packed_bytes, packed_len, win_len = workload_bytes(args.workload)
     if ragged:
-        packed_len, win_len = ragged_lengths(args.workload, b)
-        per_tok = h_k * 128 * 2
-        packed_bytes = int(packed_len.sum().item() * per_tok * (bits / 8 + 4 / gs))
-        total_bytes = packed_bytes + int(win_len.sum().item()) * per_tok * 2 + 2 * b * h * 128 * 2
         packed_dev, win_dev = packed_len.to(dev), win_len.to(dev)
-    else:
-        total_bytes, packed_bytes = algorithmic_bytes(b, h, h_k, S, R, bits, gs)
 
-    # enough distinct caches that consecutive steps cannot be served from the Infinity Cache
-    nbuf = 1 if args.no_rotate else max(2, math.ceil(320e6 / total_bytes))
-    nbuf = min(nbuf, 16)
-    plans, keep, srcs = [], [], []
-    q0 = k0 = v0 = None
-    for i in range(nbuf):
-        q, k, v = make_inputs(b, h, h_k, S + R, seed=i, dtype=dtype)
-        if i == 0:
-            q0, k0, v0 = q, k, v
-        kd, vd = k.to(dev), v.to(dev)
-        cache = alloc_cache(b, S, h_k, bits, gs, dev)
-        kvcache_pack_int(kd[:, :S], cache[0], cache[1], vd[:, :S], cache[2], cache[3], None, None, S,
-                         "k-channel", gs, bits)
-        if ragged:
-            # window of sequence j: its tokens behind the packed prefix
-            kres = torch.zeros((b, R, h_k, 128), dtype=dtype, device=dev)
-            vres = torch.zeros_like(kres)
-            for j in range(b):
-                p0, r0 = int(packed_len[j]), int(win_len[j])
-                kres[j, :r0], vres[j, :r0] = kd[j, p0:p0 + r0], vd[j, p0:p0 + r0]
-            plan = plan_fwd_kvcache_int(q.to(dev), *cache, None, scale, "k-channel", gs, bits,
-                                        seqlens_k=packed_dev, max_seqlen_k=int(packed_len.max()),
-                                        k_residual=kres, v_residual=vres, residual_len=win_dev,
-                                        max_residual_len=int(win_len.max()), num_splits=args.num_splits)
-        else:
-            kres, vres = kd[:, S:].contiguous(), vd[:, S:].contiguous()
-            plan = plan_fwd_kvcache_int(q.to(dev), *cache, None, scale, "k-channel", gs, bits,
-                                        k_residual=kres, v_residual=vres, num_splits=args.num_splits)
-        plans.append(plan)
-        keep.append((cache, kres, vres))
-        if not args.no_qpack and (i < 2 or sum(a.numel() + b_.numel() for a, b_ in srcs) * 2 < 640e6):
-            # fp16 sources for the quantize-pack leg: at least two, and enough of them (more than twice the
-            # 256 MB Infinity Cache in total) that no pack call finds its input cached
-            srcs.append((kd, vd))
-        del kd, vd
-    torch.cuda.synchronize(dev)
+    W = build_workload(args.workload, args.num_splits, no_rotate=args.no_rotate, want_sources=not args.no_qpack,
+                       cpu_inputs=True)
+    nbuf, plans, keep, srcs = W["nbuf"], W["plans"], W["keep"], W["srcs"]
+    q0, k0, v0 = W["first_inputs"]
 
     def step(i):
         plans[i % nbuf].run()
@@ -324,23 +484,14 @@ def main():
         result["us_per_step_quantiles"] = T["quantiles"]
 
     if not args.no_probe:
-        # what the memory system alone allows: a kernel that only reads as many bytes as one step streams
-        # (same launch shape, buffers rotated like the caches), timed the same way
-        import ctypes
-        from bitladder_amd import _lib
-        L = _lib.lib()
-        probe_bytes = (total_bytes + 4095) // 4096 * 4096
-        probe_bufs = [torch.randint(0, 255, (probe_bytes,), dtype=torch.uint8, device=dev) for _ in range(nbuf)]
-
-        def probe(i):
-            buf = probe_bufs[i % nbuf]
-            _lib.check(L.bitdecode_read_probe(buf.data_ptr(), probe_bytes, None, torch.cuda.current_stream(dev).cuda_stream))
-
-        us_probe = time_steps(probe, args.steps, args.warmup, not args.no_graph)["event_us"]
-        result["roofline"]["read_kernel_us"] = round(us_probe, 3)
+        # what the memory system alone allows: kernels that only read as many bytes as one step streams (buffers
+        # rotated like the caches), timed the same way; the fastest of a few launch shapes counts
+        us_probe, probe_cfg, probe_all, probe_bytes = best_probe(total_bytes, args.steps, args.warmup, not args.no_graph, nbuf)
+        result["roofline"]["read_kernel_us"] = us_probe
         result["roofline"]["read_kernel_GBs"] = round(probe_bytes / (us_probe * 1e-6) / 1e9, 1)
+        result["roofline"]["read_kernel"] = probe_cfg
+        result["roofline"]["read_kernels_tried_us"] = probe_all
         result["roofline"]["frac_of_read_kernel"] = round(us_probe / us_step_ev, 4)
-        del probe_bufs
 
     # the call a user of the reference makes: plain fwd_kvcache_int(...), eager launches, workspace from the
     # per-stream cache (nothing allocated or filled after the first call), output buffer passed in
@@ -419,6 +570,29 @@ def main():
             "entry": "bitdecode_fwd_append", "us_per_step": round(us_append, 3),
             "window_tokens": "65-%d" % (64 + math.ceil((nodes + args.warmup + 1) / n_slots)), "does": "attend + store the new token + advance the device-side length"}
         del splans
+        # the step that fills the window (one in 128): every slot starts one token short of a full window, so each
+        # step of a replay attends, stores the token, quantize-packs the 128-token window behind the prefix and
+        # advances the length; one slot per step of the graph (the slots share the rotated caches: their steps pack
+        # the same block one after the other)
+        f_slots = nodes
+        fill_start = (packed_dev - 1) if ragged else torch.full((b,), S - 1, device=dev)
+        fl_all = fill_start.to(torch.int32).repeat(f_slots, 1).contiguous()
+        fl_init = fl_all.clone()
+        fplans_ = []
+        for i in range(f_slots):
+            cache, kres, vres = keep[i % nbuf]
+            q_t = torch.randn((b, 1, h, 128), device=dev).to(dtype)
+            kn = torch.randn((b, 1, h_k, 128), device=dev).to(dtype)
+            fplans_.append(plan_fwd_kvcache_int_append(q_t, kn, kn.clone(), *cache, kres[:, :128].clone(),
+                                                       vres[:, :128].clone(), fl_all[i], S - 1, None, scale, "k-channel",
+                                                       gs, bits, num_splits=args.num_splits))
+        us_fill = time_steps(lambda i: fplans_[i % f_slots].run(), args.steps, min(args.warmup, 5), not args.no_graph,
+                             replay_prologue=lambda: fl_all.copy_(fl_init))["event_us"]
+        result["decode_step_with_append"]["fill_us_per_step"] = round(us_fill, 3)
+        result["decode_step_with_append"]["fill_does"] = ("the same launch on the step that fills the 128-token window: "
+                                                          "also quantize-packs it behind the prefix (packed prefix "
+                                                          "128 tokens shorter, window 127 + the new token)")
+        del fplans_
 
     if not args.no_fp16:
         # fp16-KV decode on the same GPU: the library's own fp16 split-KV path over all S+R tokens,
@@ -453,6 +627,26 @@ def main():
             "kernel": "same library, fp16 split-KV path", "speedup_of_low_bit": round(us16 / us_step_ev, 3),
             "torch_sdpa_us_per_step": None if us_sdpa is None else round(us_sdpa, 3)}
         del fplans
+
+    if not args.no_others and args.workload == DEFAULT_WORKLOAD and args.num_splits == 0 and not args.no_rotate:
+        # the other BASELINE shapes, compactly: inputs generated on the GPU, same timing method, read probe beside
+        others = {}
+        for name in OTHER_CONFIGS:
+            Wo = build_workload(name, 0, cpu_inputs=False, max_bufs=8)
+            n_o, plans_o = Wo["nbuf"], Wo["plans"]
+            us_o = time_steps(lambda i, n_o=n_o, plans_o=plans_o: plans_o[i % n_o].run(), args.steps, args.warmup,
+                              not args.no_graph)["event_us"]
+            entry = {"us_per_step": round(us_o, 3), "algorithmic_bytes": Wo["total_bytes"],
+                     "GB/s": round(Wo["total_bytes"] / us_o / 1e3, 1),
+                     "frac": round(Wo["total_bytes"] / us_o / 1e3 / HBM_PEAK_GBS, 4),
+                     "num_splits": plans_o[0].num_splits, "kv_buffers_rotated": n_o}
+            if not args.no_probe:
+                up, cfg, _, _ = best_probe(Wo["total_bytes"], args.steps, args.warmup, not args.no_graph, n_o)
+                entry["read_kernel_us"], entry["read_kernel"] = up, cfg
+            others[name] = entry
+            del Wo, plans_o
+            torch.cuda.empty_cache()
+        result["other_configs"] = others
 
     if not args.no_cpu and ragged:
         print("[bench] the CPU baseline leg runs on the uniform workloads only", file=sys.stderr)

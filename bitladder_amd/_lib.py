@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbitdecode.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 FP16, BF16 = 0, 1
 K_CHANNEL, K_TENSOR = 0, 1
 
@@ -71,7 +71,7 @@ class FwdAppendArgs(ctypes.Structure):
 
 EXPORTS = ("bitdecode_abi_version", "bitdecode_last_error", "bitdecode_num_splits",
            "bitdecode_fwd_workspace_bytes", "bitdecode_num_splits_for", "bitdecode_qpack", "bitdecode_fwd",
-           "bitdecode_fwd_append", "bitdecode_fwd_append_workspace_bytes", "bitdecode_read_probe", "bitdecode_fwd_static")
+           "bitdecode_fwd_append", "bitdecode_fwd_append_workspace_bytes", "bitdecode_fwd_static")
 
 _lib = None
 
@@ -112,8 +112,6 @@ def lib():
         L.bitdecode_fwd_append.argtypes = [ctypes.POINTER(FwdAppendArgs), _vp]
         L.bitdecode_fwd_append_workspace_bytes.restype = ctypes.c_size_t
         L.bitdecode_fwd_append_workspace_bytes.argtypes = [_i32] * 3
-        L.bitdecode_read_probe.restype = ctypes.c_int
-        L.bitdecode_read_probe.argtypes = [_vp, ctypes.c_size_t, _vp, _vp]
         if L.bitdecode_abi_version() != ABI_VERSION:
             raise ImportError("libbitdecode.so ABI version mismatch; rebuild it")
         _lib = L

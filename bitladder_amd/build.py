@@ -10,6 +10,8 @@ import sys
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libbitdecode.so")
+# measurement aid of the benchmark (read-only kernels); not part of the decode path, loaded by bench.py only
+PROBE_LIB_PATH = os.path.join(_HERE, "libbitdecode_probe.so")
 
 ARCH = "gfx950"
 COMMON = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
@@ -24,8 +26,8 @@ PER_FILE = {
     "qpack.hip": ["-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"],
     "decode.hip": ["-mllvm", "-amdgpu-sched-strategy=gcn-max-ilp", "-fhip-fp32-correctly-rounded-divide-sqrt"],
     "api.hip": [],
-    "probe.hip": [],
 }
+PROBE_SRC = "probe.hip"
 
 
 def hipcc() -> str:
@@ -49,12 +51,17 @@ def check_no_scratch(src: str, report: str) -> None:
 
 
 def build(verbose: bool = False) -> str:
-    """Compile every HIP source and link the shared library; returns its path."""
+    """Compile every HIP source and link the shared library (and the benchmark's probe library); returns the
+    path of the former."""
     cc = hipcc()
     objdir = os.path.join(_HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = []
     procs = []
+    probe_cmd = [cc, *COMMON, "-shared", os.path.join(CSRC, PROBE_SRC), "-o", PROBE_LIB_PATH]
+    if verbose:
+        print(" ".join(probe_cmd), flush=True)
+    probe_proc = subprocess.Popen(probe_cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     for src, extra in PER_FILE.items():
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
         cmd = [cc, *COMMON, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
@@ -67,6 +74,9 @@ def build(verbose: bool = False) -> str:
         if p.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
         check_no_scratch(src, out)
+    out, _ = probe_proc.communicate()
+    if probe_proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {PROBE_SRC}:\n{out}")
     cmd = [cc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:

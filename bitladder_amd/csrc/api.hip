@@ -401,14 +401,6 @@ int bitdecode_fwd_append(const bitdecode_fwd_append_args* a, void* stream) {
     return run_fwd(&a->fwd, a, stream);
 }
 
-int bitdecode_read_probe(const void* src, size_t bytes, void* sink, void* stream) {
-    if (!src || bytes % 16 || !aligned16(src)) return fail(BITDECODE_EINVAL, "read probe: 16-byte aligned buffer of a multiple of 16 bytes");
-    if (bytes == 0) return BITDECODE_OK;
-    hipError_t e = bitdecode::launch_read_probe(src, bytes, static_cast<unsigned int*>(sink), query_cus(), static_cast<hipStream_t>(stream));
-    if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "read probe launch failed: %s", hipGetErrorString(e));
-    return BITDECODE_OK;
-}
-
 #ifdef BITDECODE_PROF
 int bitdecode_prof_set(void* p) { return bitdecode::set_prof_buffer(static_cast<unsigned long long*>(p)) != hipSuccess; }
 #endif

@@ -49,8 +49,18 @@
 #define X_DEPTH 4
 #endif
 
+// cross-split protocol under test: 0 = stores, acknowledgement, ticket, loads; 1 = stores, ticket, validated loads;
+// 2 = ticket drawn before the workgroup's own merge, validated loads
+#ifndef X_PROTO
+#define X_PROTO 0
+#endif
+
 namespace bitdecode {
 namespace {
+
+#ifdef X_POLLSTAT
+__device__ unsigned long long g_polls[4] = {0, 0, 0, 0};
+#endif
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
@@ -1032,7 +1042,12 @@ __device__ __forceinline__ uint32_t ld_dev1_at(const uint32_t* base, uint32_t la
 __device__ __forceinline__ uint32_t pack_partial(float O0, float O1, float L) {
     const float inv = L > 0.0f ? __builtin_amdgcn_rcpf(L) : 0.0f;
     const _Float16 a = static_cast<_Float16>(O0 * inv), b = static_cast<_Float16>(O1 * inv);
-    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, a)) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, b)) << 16);
+    const uint32_t w = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, a)) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, b)) << 16);
+#if X_PROTO >= 1
+    return w ? w : 0x80000000u;      // an all-zero word means "not written yet": (+0, +0) travels as (+0, -0)
+#else
+    return w;
+#endif
 }
 __device__ __forceinline__ float partial_lo(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w))); }
 __device__ __forceinline__ float partial_hi(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16))); }
@@ -1095,11 +1110,16 @@ __device__ __forceinline__ void load_partials(uint32_t (&v)[N], const uint32_t* 
 // the additions is fixed: even and odd splits of a block are summed separately (two dependent chains instead of
 // one) and added at the end.  On return O0, O1 are the weighted sums and L the sum of the weights (the head's
 // softmax denominator relative to M).  The partial-output area is below 2^31 bytes (checked by the host).
+// Polls of a record that was not there yet, at most: its writer issued the stores before it drew its ticket, so
+// they are on their way and arrive whatever else happens; the bound only keeps a broken workspace from hanging
+// the launch.
+constexpr int kMaxPolls = 1 << 16;
+
 template <int N>
-__device__ __forceinline__ void merge_splits_n(const uint32_t* o_part, const float* ml_part, int64_t hrow,
+__device__ __forceinline__ void merge_splits_n(uint32_t* o_part, float* ml_part, int64_t hrow,
                                                int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
-    const uint32_t* head_base = o_part + hrow * nsplit * kPartialWords;
-    const float* mlb = ml_part + hrow * nsplit * 2;
+    uint32_t* head_base = o_part + hrow * nsplit * kPartialWords;
+    float* mlb = ml_part + hrow * nsplit * 2;
     const uint32_t lane_bytes = lane * 4, ml_lane = (lane & 31) * 8;
     const int sl = lane & 31;
     const float2 none = float2{-INFINITY, 0.0f};
@@ -1108,12 +1128,44 @@ __device__ __forceinline__ void merge_splits_n(const uint32_t* o_part, const flo
     float lacc = 0.0f, Mu = 0.0f;
     float e0 = 0.0f, e1 = 0.0f, d0 = 0.0f, d1 = 0.0f;
     for (int s0 = 0; s0 < nsplit; s0 += 32) {
+#if X_PROTO >= 1 && !defined(X_NOZERO)
+        for (int spin = 0;; ++spin) {
+            if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
+            load_partials<N>(v, head_base, lane_bytes, s0, nsplit);
+            uint32_t mn = v[0];
+#pragma unroll
+            for (int k = 1; k < N; ++k) mn = min(mn, v[k]);
+            bool ok = mn != 0;
+            if (s0 + sl < nsplit) ok = ok && (__float_as_uint(ml.x) | __float_as_uint(ml.y)) != 0;
+            if (__builtin_amdgcn_ballot_w64(!ok) == 0 || spin >= kMaxPolls) break;
+#ifdef X_POLLSTAT
+            if (lane == 0) atomicAdd(&g_polls[0], 1ull);
+#endif
+        }
+#ifdef X_POLLSTAT
+        if (lane == 0) atomicAdd(&g_polls[1], 1ull);
+#endif
+#else
         if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
         load_partials<N>(v, head_base, lane_bytes, s0, nsplit);
+#endif
         if (s0 == 0) {
             float mx = ml.x;
             for (int s = 32; s < nsplit; s += 32) {        // more than 32 splits: the other maxima
+#if X_PROTO >= 1 && !defined(X_NOZERO)
+                float2 t = none;
+                for (int spin = 0;; ++spin) {
+                    bool ok = true;
+                    if (s + sl < nsplit) {
+                        t = ld_dev2_at(mlb + 2 * s, ml_lane);
+                        ok = (__float_as_uint(t.x) | __float_as_uint(t.y)) != 0;
+                    }
+                    if (__builtin_amdgcn_ballot_w64(!ok) == 0 || spin >= kMaxPolls) break;
+                }
+                mx = fmaxf(mx, t.x);
+#else
                 if (s + sl < nsplit) mx = fmaxf(mx, ld_dev2_at(mlb + 2 * s, ml_lane).x);
+#endif
             }
             M = wave_max(mx);
             Mu = (M == -INFINITY) ? 0.0f : M;
@@ -1128,6 +1180,18 @@ __device__ __forceinline__ void merge_splits_n(const uint32_t* o_part, const flo
             d0 = __builtin_fmaf(wb, partial_lo(v[k + 1]), d0);
             d1 = __builtin_fmaf(wb, partial_hi(v[k + 1]), d1);
         }
+#if X_PROTO >= 1 && !defined(X_NOZERO)
+        // the records are consumed: back to "not written" for the next launch on this workspace
+        {
+            uint32_t* base = head_base + s0 * kPartialWords + lane;
+            const int cnt = nsplit - s0;
+#pragma unroll
+            for (int k = 0; k < N; ++k) {
+                if (k < cnt) st_dev1(base + k * kPartialWords, 0u);
+            }
+            if (lane < 32 && s0 + sl < nsplit) st_dev2(mlb + 2 * (s0 + sl), 0.0f, 0.0f);
+        }
+#endif
     }
     O0 = e0 + d0;
     O1 = e1 + d1;
@@ -1135,7 +1199,7 @@ __device__ __forceinline__ void merge_splits_n(const uint32_t* o_part, const flo
     const float lrow = row_sum16(lacc);
     L = lane_value(lrow, 0) + lane_value(lrow, 16);
 }
-__device__ __forceinline__ void merge_splits(const uint32_t* o_part, const float* ml_part, int64_t hrow,
+__device__ __forceinline__ void merge_splits(uint32_t* o_part, float* ml_part, int64_t hrow,
                                              int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
     // as many loads per lane as there are splits, rounded up to 4, 8, 16 or 32: every one of them is a round trip
     // of its own to the memory side (with 32 loads for 8 splits the 4K-token step took 0.5 us longer)
@@ -1300,7 +1364,7 @@ __device__ __forceinline__ int sequence_of_position(const FwdParams& P, int p, i
 template <int BITS, int GS, bool FEW>
 constexpr int fwd_lds_bytes() {
     using C = UnitCfg<BITS, GS, FEW>;
-    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16;
+    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16 + kMaxGroupHeads * 4;
 }
 
 template <int BITS, int GS, bool BF16, bool APPEND, bool KT, bool FEW>
@@ -1314,6 +1378,8 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     float* const sM = reinterpret_cast<float*>(sq + (kMaxGroupHeads + 1) * kQRowBytes);   // [8][NW]
     float* const sL = sM + NW * kMaxGroupHeads;
     int* const s_last = reinterpret_cast<int*>(sL + NW * kMaxGroupHeads);
+    int* const s_tick = s_last + 4;       // [8] tickets drawn for the heads of the group, -1 = not yet
+    if (threadIdx.x < kMaxGroupHeads) s_tick[threadIdx.x] = -1;      // (read after the workgroup barrier of the tail)
 
     PROF_DECL;
     PROF(0);
@@ -1523,6 +1589,18 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     const int hq = hk * g + wave;                                  // this wave's query head
     const int64_t hrow = static_cast<int64_t>(bi) * n_h + hq;      // its row in [b][h] tables
     uint16_t* const out_row = out + bi * out_sb + hq * out_sh;
+#if X_PROTO == 2
+    // The ticket of a head is drawn as soon as the workgroup is past its barrier, by a wave that has nothing else
+    // to do (wave g + j for head j), while the head's own wave merges and publishes: whoever holds the last
+    // ticket knows that every other split of the head has all its waves done and will publish without waiting
+    // for anybody.  The ticket travels through LDS.
+    const bool helpers = NW >= 2 * g && P.nsplit > 1;
+    if (helpers && wave >= g && wave < 2 * g && lane == 0) {
+        const int64_t hr = static_cast<int64_t>(bi) * n_h + hk * g + (wave - g);
+        const int d = __hip_atomic_fetch_add(&tickets[hr * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&s_tick[wave - g], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+#endif
     if (wave < g) {
         // weights of the waves: lane (any row, w) takes wave w; the row reductions give every lane the
         // head's maximum, the weights travel to all lanes as scalars
@@ -1545,11 +1623,27 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
             write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
         } else {
             st_dev1(&o_part[(hrow * P.nsplit + split) * kPartialWords + lane], pack_partial(O0, O1, L));
+#if X_PROTO >= 1
+            // (max, sum) is never two zero words: a zero maximum travels as -0
+            if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M == 0.0f ? -0.0f : M, L);
+            asm volatile("" ::: "memory");
+#else
             if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M, L);
             wait_vm<0>();
+#endif
             PROF(5);
             int drawn = 0;
+#if X_PROTO == 2
+            if (helpers) {
+                do {
+                    drawn = __hip_atomic_load(&s_tick[wave], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                } while (drawn < 0);
+            } else if (lane == 0) {
+                drawn = __hip_atomic_fetch_add(&tickets[hrow * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#else
             if (lane == 0) drawn = __hip_atomic_fetch_add(&tickets[hrow * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
             drawn = __builtin_amdgcn_readfirstlane(drawn);
             last = drawn == P.nsplit - 1;
             if (last && lane == 0) __hip_atomic_store(&tickets[hrow * kTicketStride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1636,6 +1730,15 @@ hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
 }
 
 }  // namespace
+
+#ifdef X_POLLSTAT
+extern "C" int bitdecode_debug_polls(unsigned long long* out4) {
+    hipError_t e = hipMemcpyFromSymbol(out4, HIP_SYMBOL(g_polls), sizeof(g_polls));
+    unsigned long long z[4] = {0, 0, 0, 0};
+    if (e == hipSuccess) e = hipMemcpyToSymbol(HIP_SYMBOL(g_polls), z, sizeof(z));
+    return e != hipSuccess;
+}
+#endif
 
 #ifdef BITDECODE_PROF
 hipError_t set_prof_buffer(unsigned long long* p) {

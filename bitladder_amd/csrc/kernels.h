@@ -84,7 +84,6 @@ inline uint32_t division_magic(uint32_t d) { return d <= 1 ? 0u : static_cast<ui
 
 hipError_t launch_qpack(const QpackParams& p, hipStream_t stream);
 hipError_t launch_fwd(const FwdParams& p, hipStream_t stream);
-hipError_t launch_read_probe(const void* src, size_t bytes, unsigned int* sink, int workgroups, hipStream_t stream);
 #ifdef BITDECODE_PROF
 hipError_t set_prof_buffer(unsigned long long* p);   // per-wave timeline buffer (tuning builds only)
 #endif

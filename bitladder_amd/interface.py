@@ -192,10 +192,18 @@ def _run_kept(key, q, kwargs, make_plan):
     memory: the validated argument block of a thread's last distinct calls (up to 512) is kept and found again by the
     address, shape, strides and element type of every tensor, which saves 40 % of the host's time per call."""
     return_lse = kwargs.get("return_lse", False)
+    if q.is_cuda and torch.cuda.is_current_stream_capturing():
+        # Recorded into a HIP graph: the graph bakes the workspace address in and may be replayed on any stream,
+        # at any time.  The call gets a workspace of its own, allocated (and zero-filled by a fill kernel) inside
+        # the capture, so it lives in the graph's memory pool for as long as the graph does; none of the caches is used.
+        plan = make_plan(False)
+        with _on_device(plan.device):
+            plan.run()
+        return (plan.out, plan.lse) if return_lse else plan.out
     cache = _plan_cache()
     plan = cache.get(key)
     if plan is None:
-        plan = make_plan()
+        plan = make_plan(True)
         out, lse = plan.out, plan.lse
         # a kept plan must not keep the caller's tensors alive: it holds addresses, and its workspace
         fwd = plan.args.fwd if isinstance(plan.args, _lib.FwdAppendArgs) else plan.args
@@ -464,9 +472,9 @@ def fwd_kvcache_int(q: torch.Tensor,
                     (softmax_scale, quant_mode, group_size, num_bits), kwargs)
     # the split workspace comes from a per-stream cache: no allocation and no fill after the first call
     # (the reference allocates its accumulators per call, decode_api.cpp:292-295, 375-390)
-    return _run_kept(key, q, kwargs, lambda: plan_fwd_kvcache_int(
+    return _run_kept(key, q, kwargs, lambda shared: plan_fwd_kvcache_int(
         q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale, quant_mode, group_size, num_bits,
-        _stream_ws=True, **kwargs))
+        _stream_ws=shared, **kwargs))
 
 
 def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
@@ -546,6 +554,6 @@ def fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Te
     """
     key = _call_key((q, k_new, v_new, k_pack, k_params, v_pack, v_params, k_residual, v_residual, lengths,
                      opt_block_table), ("step", max_len, softmax_scale, quant_mode, group_size, num_bits), kwargs)
-    return _run_kept(key, q, kwargs, lambda: plan_fwd_kvcache_int_append(
+    return _run_kept(key, q, kwargs, lambda shared: plan_fwd_kvcache_int_append(
         q, k_new, v_new, k_pack, k_params, v_pack, v_params, k_residual, v_residual, lengths, max_len,
-        opt_block_table, softmax_scale, quant_mode, group_size, num_bits, _stream_ws=True, **kwargs))
+        opt_block_table, softmax_scale, quant_mode, group_size, num_bits, _stream_ws=shared, **kwargs))

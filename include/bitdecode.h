@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define BITDECODE_ABI_VERSION 4
+#define BITDECODE_ABI_VERSION 5
 
 enum {
     BITDECODE_OK = 0,
@@ -178,11 +178,6 @@ int bitdecode_num_splits_for(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32
  * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,
  * csrc/bit_decode/decode_api.cpp:292-295). */
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits);
-
-/* Measurement aid (no counterpart in the reference): a kernel that only reads `bytes` bytes (a multiple of
- * 16) at `src` with the decode kernel's launch shape, one workgroup per compute unit.  bench.py times it
- * over the bytes of a decode step as the ceiling the memory system sets for that step.  `sink` may be NULL. */
-int bitdecode_read_probe(const void* src, size_t bytes, void* sink, void* stream);
 
 int bitdecode_abi_version(void);
 const char* bitdecode_last_error(void);

@@ -31,9 +31,11 @@ def _run_config(device, b, h, h_k, S, R, bits, gs, dtype, seed=0, check_batches=
     cache_np = H.cache_to_numpy(*cache)
     worst = 0.0
     g = h // h_k
-    hks = list(range(h_k)) if check_kv_heads is None else list(check_kv_heads)
-    hqs = [hk * g + j for hk in hks for j in range(g)]
     for bi in (range(b) if check_batches is None else check_batches):
+        # kv heads compared for this batch row: all, a fixed set, or a choice per row
+        hks = (list(range(h_k)) if check_kv_heads is None else
+               list(check_kv_heads(bi)) if callable(check_kv_heads) else list(check_kv_heads))
+        hqs = [hk * g + j for hk in hks for j in range(g)]
         sl = slice(bi, bi + 1)
         qkv = O.quantize_kv_ref(k[sl, :S][:, :, hks], v[sl, :S][:, :, hks], bits, gs, dtype)
         # k_pack (b, S/pn, h_k, d), k_params (b, S/gs, h_k, d), v_pack (b, S, h_k, d/pn), v_params (b, d/gs, h_k, S)
@@ -79,13 +81,14 @@ def test_c2_statistical_crosscheck_vs_unquantized(device):
 
 
 def test_c3_llama3_8b_gqa_128k_2bit_g64(device):
-    """Long split-KV partitioning and the cross-split combine; oracle on two of the eight kv heads."""
-    _run_config(device, 1, 32, 8, 131072, 128, 2, 64, "fp16", check_kv_heads=(0, 5))
+    """Long split-KV partitioning and the cross-split combine; oracle on all eight kv heads."""
+    _run_config(device, 1, 32, 8, 131072, 128, 2, 64, "fp16")
 
 
 def test_c5_llama3_70b_layer_bf16_2bit(device):
-    """b8, 64 q / 8 kv heads (group of 8), S=65536, 2-bit g128, bf16; oracle on two (batch, kv-head) pairs."""
-    _run_config(device, 8, 64, 8, 65536, 128, 2, 128, "bf16", check_batches=(0, 7), check_kv_heads=(3,))
+    """b8, 64 q / 8 kv heads (group of 8), S=65536, 2-bit g128, bf16; oracle on one kv head of every batch row
+    (a different one per row, so every kv head index is compared once)."""
+    _run_config(device, 8, 64, 8, 65536, 128, 2, 128, "bf16", check_kv_heads=lambda bi: ((3 * bi + 1) % 8,))
 
 
 def test_c4_ragged_batch_decode_and_append(device):

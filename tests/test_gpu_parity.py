@@ -392,3 +392,65 @@ def test_device_side_lengths_and_offsets_beyond_the_buffers_are_clamped(device):
         for t, t0 in zip(cache, before):
             assert torch.equal(t[1], t0[1])                  # sequence 1: nothing written
         assert not torch.equal(cache[0][0], before[0][0])    # sequence 0: its chunk was packed
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 128), (2, 128)])
+@pytest.mark.parametrize("ns", [2, 4, 32])
+def test_splits_whose_outputs_cancel_stay_within_the_bar(device, bits, gs, ns):
+    """Designed inputs: the splits' own outputs are about +5 and -5 in every channel (|v| = 4 ... 6, signs that flip
+    from one split to the next) with near-equal softmax weights, so the merged output is small and whatever the
+    partial outputs lose on their way between workgroups shows in full against the plain 2e-3 bar.  The
+    reference keeps its partial outputs in fp32 (flash_fwd_kernel.h:1280-1298)."""
+    from bitladder_amd import fwd_kvcache_int
+    b, h, h_k, S = 2, 8, 2, 128 * ns * 4
+    rng = np.random.default_rng(1234 + ns + bits)
+    q = (0.05 * rng.standard_normal((b, 1, h, 128))).astype(np.float32)      # flat softmax: weights nearly equal
+    k = rng.standard_normal((b, S, h_k, 128)).astype(np.float32)
+    sign_c = rng.choice([-1.0, 1.0], size=(1, 1, h_k, 128)).astype(np.float32)
+    sign_s = np.where((np.arange(S) // (S // ns)) % 2 == 0, 1.0, -1.0).astype(np.float32).reshape(1, S, 1, 1)
+    v = (sign_c * sign_s * (5.0 + 0.3 * rng.standard_normal((b, S, h_k, 128)))).astype(np.float32)
+    q, k, v = (O.round_to_storage(x, "fp16") for x in (q, k, v))
+    qkv = O.quantize_kv_ref(k, v, bits, gs)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, _ = O.attend_ref(q, k_hat, v_hat, SCALE)
+    assert np.abs(want).max() < 0.5, "the designed outputs are meant to cancel"
+    out = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns)
+    one = fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits, num_splits=1)
+    err = np.abs(out.float().cpu().numpy() - want).max()
+    err1 = np.abs(one.float().cpu().numpy() - want).max()
+    assert err1 < ATOL, err1
+    assert err < ATOL, (ns, err, err1)
+
+
+def test_plain_call_recorded_into_a_hip_graph_has_a_workspace_of_its_own(device):
+    """fwd_kvcache_int (not a plan) recorded into a HIP graph: the recorded call must not share the per-stream
+    workspace cache with later eager calls.  The graph is replayed on a side stream while eager calls of the same
+    shape run on the default stream, several times; every replay and every eager call reproduces its result."""
+    from bitladder_amd import fwd_kvcache_int
+    from bitladder_amd import interface as I
+    b, h, h_k, S, bits, gs, ns = 2, 8, 2, 128 * 16, 4, 128, 4
+    q, k, v = O.make_inputs(b, h, h_k, S, 0, seed=91)
+    cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+    qd = H.to_dev(q, "fp16", device)
+    q2 = (qd * -0.75).contiguous()
+    eager1 = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns).clone()
+    eager2 = fwd_kvcache_int(q2, *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns).clone()
+    torch.cuda.synchronize()
+    shared = {id(w) for w in I._WORKSPACES.values()}
+    out_g = torch.empty_like(qd)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns, out=out_g)
+    assert {id(w) for w in I._WORKSPACES.values()} == shared, "the capture must not add to the stream workspaces"
+    side = torch.cuda.Stream(device)
+    for rep in range(4):
+        out_g.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            graph.replay()
+        outs = [fwd_kvcache_int(q2, *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns) for _ in range(3)]
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, eager1), rep
+        for o in outs:
+            assert torch.equal(o, eager2), rep

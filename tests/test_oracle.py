@@ -377,3 +377,27 @@ def test_zero_minimum_takes_the_sign_of_a_negative_zero():
     assert np.signbit(a.k_zero[0, 0, 0, 3]) and not np.signbit(a.k_zero[0, 0, 0, 4])
     np.testing.assert_array_equal(np.signbit(a.k_zero), np.signbit(c.k_zero))
     np.testing.assert_array_equal(np.signbit(a.v_zero), np.signbit(c.v_zero))
+
+
+def test_round_to_bf16_equals_the_library_conversion():
+    """round_to_bf16 (the oracle's storage rounding for bf16 inputs, scales and zeros) against an independent
+    implementation: torch's fp32 -> bf16 conversion (round to nearest, ties to even), on random values over
+    the whole exponent range, on exact ties with an even and an odd neighbour below, on values around the
+    largest finite bf16, on subnormals, zeros and infinities."""
+    import torch
+    rng = np.random.default_rng(5)
+    bits = rng.integers(0, 1 << 32, size=1 << 20, dtype=np.uint64).astype(np.uint32)
+    rand = bits.view(np.float32)
+    rand = rand[np.isfinite(rand)]
+    # exact ties: upper 16 bits arbitrary, lower 16 bits = 0x8000; both parities of bit 16 occur
+    hi = rng.integers(0, 1 << 16, size=1 << 16, dtype=np.uint64).astype(np.uint32)
+    ties = ((hi << 16) | np.uint32(0x8000)).view(np.float32)
+    ties = ties[np.isfinite(ties)]
+    near = (((hi << 16) | np.uint32(0x7FFF)).view(np.float32), ((hi << 16) | np.uint32(0x8001)).view(np.float32))
+    edge = np.array([0.0, -0.0, np.inf, -np.inf, 3.3895314e38, 3.4e38, -3.4e38, 1e-40, -1e-40, 1.0, 1.00390625,
+                     1.01171875, 65504.0, 6.1e-5], dtype=np.float32)
+    x = np.concatenate([rand, ties, near[0][np.isfinite(near[0])], near[1][np.isfinite(near[1])], edge])
+    want = torch.from_numpy(x.copy()).to(torch.bfloat16).to(torch.float32).numpy()
+    got = O.round_to_bf16(x)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.isnan(O.round_to_bf16(np.array([np.nan], np.float32))[0])
