@@ -30,15 +30,29 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // Scratch of bitdecode_fwd_static: device memory that belongs to the library's code object, so the call
 // needs no allocation.  Every GPU that loads the library holds its own copy until the process ends.
 // Layout: arrival counters for up to kStaticHeads (batch x query head) rows, one 256-byte block each,
-// then the partial outputs and (max, sum) pairs of the splits.  The counter area is apart from the rest
-// for every problem size, so the zeros it is loaded with, and that every call leaves behind, hold from
-// call to call whatever the shapes.
+// then the two record slots of the splits.  Calls of different shapes follow one another on this one
+// array, and the decode kernel expects the part it uses to be zero when a shape starts on it: every
+// call therefore clears its counters and record slots with a small fill kernel in front of the decode
+// kernel (a kernel, not a memset node: the call may be recorded into a HIP graph).
 constexpr size_t kStaticHeads = 4096;
 constexpr size_t kStaticCounterBytes = kStaticHeads * bitdecode::kTicketStride * sizeof(int);     // 1 MiB
 constexpr size_t kStaticScratchBytes = size_t(8) << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 // address of `scratch` on each device (the name itself is only a host-side handle)
 unsigned char* g_scratch_ptr[64] = {};
+
+// 16-byte stores of zero over [p, p + n16 * 16)
+__global__ void zero_fill_kernel(uint4* p, size_t n16) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride) p[i] = uint4{0, 0, 0, 0};
+}
+hipError_t zero_fill(void* p, size_t bytes, hipStream_t stream) {      // bytes: a multiple of 16
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return hipSuccess;
+    const unsigned int blocks = static_cast<unsigned int>(std::min<size_t>((n16 + 255) / 256, 1024));
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<uint4*>(p), n16);
+    return hipGetLastError();
+}
 
 int check_quant(int bits, int gs, int dtype, int d) {
     if (d != bitdecode::kHeadDim) return fail(BITDECODE_EUNSUPPORTED, "head_dim %d unsupported (only 128)", d);
@@ -140,9 +154,14 @@ int bitdecode_num_splits_for(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32
 // [tickets: one 256-byte block per (batch, query head)][o_part][ml_part]
 static size_t ticket_bytes(int32_t b, int32_t h) { return static_cast<size_t>(b) * h * bitdecode::kTicketStride * sizeof(int); }
 
+// two slots of records behind the counters (kernels.h: split_slot_words)
+static size_t slots_bytes(int32_t b, int32_t h, int32_t num_splits) {
+    return 2 * bitdecode::split_slot_words(static_cast<size_t>(b) * h, static_cast<size_t>(num_splits)) * sizeof(uint32_t);
+}
+
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits) {
     if (num_splits <= 1) return 0;
-    return ticket_bytes(b, h) + static_cast<size_t>(num_splits) * b * h * (bitdecode::kPartialWords + 2) * sizeof(float);
+    return ticket_bytes(b, h) + slots_bytes(b, h, num_splits);
 }
 
 // paged cache: cache_tokens is the page size; the table must cover `tokens` per sequence
@@ -288,19 +307,23 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
     const int cus = query_cus();
     if (nsplit == 0)
         nsplit = choose_splits_for(a->b, a->h_k, max_s, max_r, cus, a->bits, a->group_size, a->seqlens_k && !step);
-    if (nsplit > 1 && static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords * sizeof(uint32_t) >= (size_t(1) << 31))
+    if (nsplit > 1 && slots_bytes(a->b, a->h, nsplit) >= (size_t(1) << 31))
         return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d heads: partial outputs of 2 GiB or more", nsplit, a->b, a->h);
     // the kernel divides workgroup ids and unit counts by the split count and the head count with a
     // multiply (kernels.h: division_magic), exact while numerator x divisor stays below 2^32
     {
         const uint64_t wgs = static_cast<uint64_t>(nsplit) * a->b * a->h_k;
-        const uint64_t units = static_cast<uint64_t>(max_s) / 64 + static_cast<uint64_t>(nsplit);
+        // lengths read on the device are clamped to the capacity by the kernel, not to max_seqlen_k: that is the bound
+        const uint64_t cap_tokens = a->block_table ? static_cast<uint64_t>(a->max_pages_per_seq) * a->cache_tokens
+                                                   : static_cast<uint64_t>(a->cache_tokens);
+        const uint64_t longest = (a->seqlens_k || step) ? std::max<uint64_t>(cap_tokens, max_s) : static_cast<uint64_t>(max_s);
+        const uint64_t units = longest / 64 + static_cast<uint64_t>(nsplit);
         if (wgs * std::max(nsplit, a->h_k) >= (1ull << 32) || units * nsplit >= (1ull << 32))
             return fail(BITDECODE_EUNSUPPORTED, "%d splits x %d x %d kv heads: too many workgroups", nsplit, a->b, a->h_k);
     }
     if (static_scratch) {
         const size_t rows = static_cast<size_t>(a->b) * a->h;
-        const size_t need = nsplit > 1 ? static_cast<size_t>(nsplit) * rows * (kPartialWords + 2) * sizeof(float) : 0;
+        const size_t need = nsplit > 1 ? slots_bytes(a->b, a->h, nsplit) : 0;
         if (rows > kStaticHeads || need > kStaticScratchBytes - kStaticCounterBytes)
             return fail(BITDECODE_EWORKSPACE, "bitdecode_fwd_static: %d splits x %zu (batch x head) rows need %zu bytes; the "
                         "built-in scratch holds %zu rows and %zu bytes (use bitdecode_fwd with a workspace)", nsplit, rows,
@@ -366,14 +389,22 @@ static int run_fwd(const bitdecode_fwd_args* a, const bitdecode_fwd_append_args*
         P.knew_sb = step->knew_stride_b; P.knew_sh = step->knew_stride_h;
         P.vnew_sb = step->vnew_stride_b; P.vnew_sh = step->vnew_stride_h;
     }
-    if (nsplit > 1 && static_scratch) {
-        P.tickets = reinterpret_cast<int*>(static_scratch);
-        P.o_part = reinterpret_cast<uint32_t*>(static_scratch + kStaticCounterBytes);
-        P.ml_part = reinterpret_cast<float*>(P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords);
-    } else if (nsplit > 1) {
-        P.tickets = reinterpret_cast<int*>(ws);
-        P.o_part = reinterpret_cast<uint32_t*>(ws + ticket_bytes(a->b, a->h));
-        P.ml_part = reinterpret_cast<float*>(P.o_part + static_cast<size_t>(nsplit) * a->b * a->h * kPartialWords);
+    if (nsplit > 1) {
+        const size_t records = static_cast<size_t>(nsplit) * a->b * a->h;
+        if (static_scratch) {
+            P.tickets = reinterpret_cast<int*>(static_scratch);
+            P.o_part = reinterpret_cast<uint32_t*>(static_scratch + kStaticCounterBytes);
+        } else {
+            P.tickets = reinterpret_cast<int*>(ws);
+            P.o_part = reinterpret_cast<uint32_t*>(ws + ticket_bytes(a->b, a->h));
+        }
+        P.ml_part = reinterpret_cast<float*>(P.o_part + 2 * records * kPartialWords);
+        if (static_scratch) {
+            // another shape may have used the array before: counters and record slots of this call start at zero
+            hipError_t e = zero_fill(P.tickets, ticket_bytes(a->b, a->h), static_cast<hipStream_t>(stream));
+            if (e == hipSuccess) e = zero_fill(P.o_part, slots_bytes(a->b, a->h, nsplit), static_cast<hipStream_t>(stream));
+            if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));
+        }
     }
     hipError_t e = launch_fwd(P, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(BITDECODE_ELAUNCH, "decode launch failed: %s", hipGetErrorString(e));

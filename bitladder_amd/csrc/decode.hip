@@ -44,23 +44,8 @@
 #include "layout.h"
 #include "qpack_chunk.h"
 
-// rows a wave keeps in flight (see "the rows of a unit as a pipeline")
-#ifndef X_DEPTH
-#define X_DEPTH 4
-#endif
-
-// cross-split protocol under test: 0 = stores, acknowledgement, ticket, loads; 1 = stores, ticket, validated loads;
-// 2 = ticket drawn before the workgroup's own merge, validated loads
-#ifndef X_PROTO
-#define X_PROTO 0
-#endif
-
 namespace bitdecode {
 namespace {
-
-#ifdef X_POLLSTAT
-__device__ unsigned long long g_polls[4] = {0, 0, 0, 0};
-#endif
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
@@ -86,7 +71,16 @@ __device__ unsigned long long* g_prof = nullptr;
             for (int i_ = 0; i_ < 16; ++i_) pb[i_] = prof_ts[i_];                                     \
         }                                                                                             \
     } while (0)
+#define PROF_AT(pts, slot)                          \
+    do {                                           \
+        __builtin_amdgcn_sched_barrier(0);         \
+        (pts)[slot] = wall_clock64();              \
+        __builtin_amdgcn_sched_barrier(0);         \
+    } while (0)
+#define PROF_TS prof_ts
 #else
+#define PROF_AT(pts, slot) do { } while (0)
+#define PROF_TS nullptr
 #define PROF_DECL do { } while (0)
 #define PROF(slot) do { } while (0)
 #define PROF_FLUSH() do { } while (0)
@@ -121,7 +115,9 @@ __device__ __forceinline__ h8 cvt_h8(u4 raw) {
 
 // n / d with the host's magic number for d (kernels.h)
 __device__ __forceinline__ int div_magic(int n, uint32_t magic) {
-    return magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(n), magic)) : n;
+    // (a select, not a branch: the index arithmetic of the prologue stays one basic block)
+    const uint32_t q = __umulhi(static_cast<uint32_t>(n), magic), keep = magic ? 0u : 0xffffffffu;
+    return static_cast<int>((q & ~keep) | (static_cast<uint32_t>(n) & keep));
 }
 
 __device__ __forceinline__ u4 ld_u4(const void* p) { return *reinterpret_cast<const u4*>(p); }
@@ -350,7 +346,7 @@ struct UnitCfg {
     static constexpr int OFF_KP = 8192, OFF_VP = 8192 + 2 * KPB;
     static constexpr int REGION = unit_region_bytes(BITS, GS);
     static constexpr int NW = FEW ? 8 : decode_waves(BITS, GS);        // waves per workgroup
-    static constexpr int WANT_DEPTH = FEW ? 6 : (X_DEPTH);
+    static constexpr int WANT_DEPTH = FEW ? 6 : 4;
     static constexpr int DEPTH = WANT_DEPTH < NKP + RPS + 1 ? WANT_DEPTH : NKP + RPS + 1;   // rows a wave keeps in flight
     static_assert(REGION == OFF_VP + VPB && REGION % 256 == 0, "region layout");
     static_assert(KPB_T <= KPB && (KPB_T + 1023) / 1024 == NKP, "the per-token K parameters use the same rows");
@@ -878,6 +874,15 @@ __device__ __forceinline__ kblock karg_block() {
                  : "=s"(v) : "s"(__builtin_amdgcn_kernarg_segment_ptr()), "n"(OFF) : "memory");
     return v;
 }
+// A value that an asm block delivered in scalar registers, told to the compiler as wave-uniform: it takes the
+// results of an asm statement for lane-dependent and would carry everything computed from them (addresses above
+// all) in vector registers.  The halves of a 64-bit value are widened as unsigned.
+__device__ __forceinline__ uint32_t uni32(uint32_t x) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(x)));
+}
+__device__ __forceinline__ uint64_t uni64(uint64_t x) {
+    return static_cast<uint64_t>(uni32(static_cast<uint32_t>(x))) | (static_cast<uint64_t>(uni32(static_cast<uint32_t>(x >> 32))) << 32);
+}
 template <int OFF, int FIELD_OFF>
 __device__ __forceinline__ uint64_t block_u64(const kblock& v) {
     static_assert(FIELD_OFF >= OFF && FIELD_OFF + 8 <= OFF + 64 && (FIELD_OFF - OFF) % 4 == 0, "field inside the block");
@@ -889,12 +894,12 @@ __device__ __forceinline__ uint32_t block_u32(const kblock& v) {
     return v[(FIELD_OFF - OFF) / 4];
 }
 #define BLOCK_AT(field) offsetof(FwdParams, field)
-#define BLOCK_PTR(type, blk, first, field) reinterpret_cast<type>(block_u64<BLOCK_AT(first), BLOCK_AT(field)>(blk))
-#define BLOCK_I64(blk, first, field) static_cast<int64_t>(block_u64<BLOCK_AT(first), BLOCK_AT(field)>(blk))
-#define BLOCK_I32(blk, first, field) static_cast<int>(block_u32<BLOCK_AT(first), BLOCK_AT(field)>(blk))
-#define LATE_I32(field) static_cast<int>(karg_u32<offsetof(FwdParams, field)>())
-#define LATE_I64(field) static_cast<int64_t>(karg_u64<offsetof(FwdParams, field)>())
-#define LATE_PTR(type, field) reinterpret_cast<type>(karg_u64<offsetof(FwdParams, field)>())
+#define BLOCK_PTR(type, blk, first, field) reinterpret_cast<type>(uni64(block_u64<BLOCK_AT(first), BLOCK_AT(field)>(blk)))
+#define BLOCK_I64(blk, first, field) static_cast<int64_t>(uni64(block_u64<BLOCK_AT(first), BLOCK_AT(field)>(blk)))
+#define BLOCK_I32(blk, first, field) static_cast<int>(uni32(block_u32<BLOCK_AT(first), BLOCK_AT(field)>(blk)))
+#define LATE_I32(field) static_cast<int>(uni32(karg_u32<offsetof(FwdParams, field)>()))
+#define LATE_I64(field) static_cast<int64_t>(uni64(karg_u64<offsetof(FwdParams, field)>()))
+#define LATE_PTR(type, field) reinterpret_cast<type>(uni64(karg_u64<offsetof(FwdParams, field)>()))
 
 // ---------------------------------------------------------------------------------------------
 // 16-token tiles of the fp16 residual window (tokens n0 .. n0+15, valid below R)
@@ -913,10 +918,10 @@ struct WindowSrc {
     const uint16_t* kn;
     const uint16_t* vn;
 };
-template <bool APPEND>
+template <bool APPEND, bool LATE>
 __device__ __forceinline__ WindowSrc window_src(const FwdParams& P, int bi, int hk) {
     WindowSrc W;
-    if constexpr (!APPEND) {
+    if constexpr (!LATE) {
         W.kr = P.k_res + bi * P.kres_sb + hk * P.kres_sh;
         W.vr = P.v_res + bi * P.vres_sb + hk * P.vres_sh;
         W.k_st = P.kres_st;
@@ -1031,26 +1036,40 @@ __device__ __forceinline__ float2 ld_dev2(const float* p) {
 __device__ __forceinline__ void st_dev1(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ uint32_t ld_dev1_at(const uint32_t* base, uint32_t lane_bytes) {
-    return __hip_atomic_load(reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes),
-                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 // A split's partial output as it crosses workgroups: normalised (O / L: a weighted mean of V rows, so inside the
-// value range of V whatever the split's length) and rounded to nearest fp16, two channels per 32-bit word.
-// Half the bytes of fp32 partials: the workgroup that merges reads g x splits of them through one compute
-// unit's memory path, which is what its time goes into (32 splits of 4 heads: 0.45 us less per step).
-__device__ __forceinline__ uint32_t pack_partial(float O0, float O1, float L) {
-    const float inv = L > 0.0f ? __builtin_amdgcn_rcpf(L) : 0.0f;
-    const _Float16 a = static_cast<_Float16>(O0 * inv), b = static_cast<_Float16>(O1 * inv);
+// value range of V whatever the split's length) and rounded to nearest fp16, two channels per 32-bit word: half
+// the bytes of fp32 partials for the workgroup that merges g x splits of them through one compute unit's memory
+// path.  The rounding is at most 2^-11 of the value; a split whose output reaches 2 in some channel (so that the
+// rounding could exceed 4.9e-4) also sends the residuals `lo` = value - hi, again as fp16 (22 significant bits
+// together), which the merging wave adds: splits of large outputs that cancel stay inside the error bar (the
+// reference keeps its partial outputs in fp32, flash_fwd_kernel.h:1280-1298).
+// An all-zero word means "not written": (+0, +0) travels as (+0, -0), which adds up to the same sums.
+__device__ __forceinline__ uint32_t pack_h2_nonzero(_Float16 a, _Float16 b) {
     const uint32_t w = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, a)) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, b)) << 16);
-#if X_PROTO >= 1
-    return w ? w : 0x80000000u;      // an all-zero word means "not written yet": (+0, +0) travels as (+0, -0)
-#else
-    return w;
-#endif
+    return w ? w : 0x80000000u;
 }
-__device__ __forceinline__ float partial_lo(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w))); }
-__device__ __forceinline__ float partial_hi(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16))); }
+struct PartialWords {
+    float n0, n1;      // the normalised values
+    _Float16 a, b;     // ... rounded
+    __device__ __forceinline__ PartialWords(float O0, float O1, float L) {
+        const float inv = L > 0.0f ? __builtin_amdgcn_rcpf(L) : 0.0f;
+        n0 = O0 * inv;
+        n1 = O1 * inv;
+        a = static_cast<_Float16>(n0);
+        b = static_cast<_Float16>(n1);
+    }
+    __device__ __forceinline__ uint32_t hi() const { return pack_h2_nonzero(a, b); }
+    __device__ __forceinline__ uint32_t lo() const {
+        return pack_h2_nonzero(static_cast<_Float16>(n0 - static_cast<float>(a)), static_cast<_Float16>(n1 - static_cast<float>(b)));
+    }
+    // some lane's value reaches the magnitude from which the residual words are sent
+    __device__ __forceinline__ bool large(float from) const {
+        return __builtin_amdgcn_ballot_w64(fmaxf(__builtin_fabsf(n0), __builtin_fabsf(n1)) >= from) != 0;
+    }
+};
+constexpr float kPartialLoFrom = 2.0f;      // a split sends the residual words from this output magnitude on
+__device__ __forceinline__ float half_lo(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w))); }
+__device__ __forceinline__ float half_hi(uint32_t w) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16))); }
 
 // x of lane `l` (wave-uniform index) as a scalar
 __device__ __forceinline__ float lane_value(float x, int l) {
@@ -1081,136 +1100,157 @@ __device__ __forceinline__ float wave_max(float x) {
     return fmaxf(fmaxf(lane_value(x, 0), lane_value(x, 16)), fmaxf(lane_value(x, 32), lane_value(x, 48)));
 }
 
-// 8 bytes per lane at (wave-uniform base) + (32-bit lane offset): the base stays in scalar registers, so a
-// run of such loads costs two scalar additions per load and no vector address arithmetic
+// 8 bytes per lane at (wave-uniform base) + (32-bit lane offset): the base stays in scalar registers
 __device__ __forceinline__ float2 ld_dev2_at(const float* base, uint32_t lane_bytes) {
     return ld_dev2(reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes));
 }
+
+// 4 bytes per lane at (wave-uniform base) + (32-bit lane offset), device scope
+__device__ __forceinline__ uint32_t ld_dev1_at(const uint32_t* base, uint32_t lane_bytes) {
+    return __hip_atomic_load(reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(base) + lane_bytes),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 // partial outputs (two channels per lane, 4 bytes) of splits s0 .. s0+N-1 of one query head.  The splits of a
-// head lie 256 bytes apart, so a full block of N loads differs only in the instruction's immediate offset and is
-// issued back to back; past the last split the last one is read again (its weight is zero).
+// head lie 256 bytes apart, so the N loads differ only in the instruction's immediate offset and are issued back to
+// back.  Past the head's last split the loads run on into the records behind it (the next head's, or the residual
+// words that follow the partial outputs: the area behind the last head is longer than N records); the caller
+// replaces what they return (settle_partials).
 template <int N>
-__device__ __forceinline__ void load_partials(uint32_t (&v)[N], const uint32_t* head_base, uint32_t lane_bytes,
-                                              int s0, int nsplit) {
+__device__ __forceinline__ void load_partials(uint32_t (&v)[N], const uint32_t* head_base, uint32_t lane_bytes, int s0) {
     const uint32_t* base = head_base + s0 * kPartialWords;
-    const int cnt = nsplit - s0;
-    if (cnt >= N) {
 #pragma unroll
-        for (int k = 0; k < N; ++k) v[k] = ld_dev1_at(base + k * kPartialWords, lane_bytes);
-    } else {
+    for (int k = 0; k < N; ++k) v[k] = ld_dev1_at(base + k * kPartialWords, lane_bytes);
+}
+// words of splits that do not exist: a valid pair of ones (their weight is zero)
+template <int N>
+__device__ __forceinline__ void settle_partials(uint32_t (&v)[N], int cnt) {
+    if (cnt < N) {
 #pragma unroll
-        for (int k = 0; k < N; ++k) v[k] = ld_dev1_at(base + (k < cnt ? k : cnt - 1) * kPartialWords, lane_bytes);
+        for (int k = 0; k < N; ++k) v[k] = k < cnt ? v[k] : 0x3c003c00u;
     }
 }
+
+// Polls of a record that was not there yet, at most.  Every writer of a record the merging wave waits for has
+// passed its workgroup's barrier and publishes without waiting for anybody, so the records arrive whatever else
+// happens; the bound only keeps a misused workspace from hanging the launch.
+constexpr int kMaxPolls = 1 << 16;
 
 // Merge of the splits of one query head by one wave (flash_fwd_kernel.h:1217-1298 with normalised partials):
 // out = sum_s w_s O_s / sum_s w_s with w_s = 2^(M_s - max M) L_s and O_s the split's normalised output.
 // Lane l owns channels 2l and 2l+1.  Splits are taken N at a time (N = 32, or less when there are fewer splits):
-// lane l holds the (M, L) pair of split s0 + l % 32, the weights go back to all lanes as scalars.  The order of
-// the additions is fixed: even and odd splits of a block are summed separately (two dependent chains instead of
-// one) and added at the end.  On return O0, O1 are the weighted sums and L the sum of the weights (the head's
-// softmax denominator relative to M).  The partial-output area is below 2^31 bytes (checked by the host).
-// Polls of a record that was not there yet, at most: its writer issued the stores before it drew its ticket, so
-// they are on their way and arrive whatever else happens; the bound only keeps a broken workspace from hanging
-// the launch.
-constexpr int kMaxPolls = 1 << 16;
-
-template <int N>
-__device__ __forceinline__ void merge_splits_n(uint32_t* o_part, float* ml_part, int64_t hrow,
-                                               int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
+// lane l holds the (M, L) pair of split s0 + l % 32, the weights go back to all lanes as scalars.  A record is
+// valid when none of its words is zero; the loads of a block are repeated while one still reads "not written".
+// A split that sent residual words (negative sum) has them added with the same weight.  The order of the
+// additions is fixed: even and odd splits of a block are summed separately (two dependent chains instead of
+// one) and added at the end, so the result does not depend on timing.  On return O0, O1 are the weighted sums
+// and L the sum of the weights (the head's softmax denominator relative to M).  The partial-output area is
+// below 2^31 bytes (checked by the host).
+template <int N, int BLOCK>
+__device__ __forceinline__ void merge_splits_n(uint32_t* o_part, uint32_t lo_words, float* ml_part, int64_t hrow,
+                                               int nsplit, int lane, float& O0, float& O1, float& M, float& L, [[maybe_unused]] unsigned long long* pts = nullptr) {
     uint32_t* head_base = o_part + hrow * nsplit * kPartialWords;
     float* mlb = ml_part + hrow * nsplit * 2;
-    const uint32_t lane_bytes = lane * 4, ml_lane = (lane & 31) * 8;
-    const int sl = lane & 31;
-    const float2 none = float2{-INFINITY, 0.0f};
-    uint32_t v[N];
-    float2 ml = none;
+    const uint32_t lane_bytes = lane * 4;
+    static_assert((BLOCK == 32 || BLOCK == 16) && N <= BLOCK, "splits per block");
+    const int sl = lane & (BLOCK - 1);
     float lacc = 0.0f, Mu = 0.0f;
     float e0 = 0.0f, e1 = 0.0f, d0 = 0.0f, d1 = 0.0f;
-    for (int s0 = 0; s0 < nsplit; s0 += 32) {
-#if X_PROTO >= 1 && !defined(X_NOZERO)
+    for (int s0 = 0; s0 < nsplit; s0 += BLOCK) {
+        const bool mine = s0 + sl < nsplit;
+        const uint32_t ml_lane = static_cast<uint32_t>(min(s0 + sl, nsplit - 1)) * 8;
+        const float se0 = e0, se1 = e1, sd0 = d0, sd1 = d1;
+        float2 ml;
+        float w;
+        // One flight of loads per attempt; the words are checked as they are used (none of them may be zero), and an
+        // attempt that met a record still "not written" is thrown away and repeated.
         for (int spin = 0;; ++spin) {
-            if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
-            load_partials<N>(v, head_base, lane_bytes, s0, nsplit);
-            uint32_t mn = v[0];
-#pragma unroll
-            for (int k = 1; k < N; ++k) mn = min(mn, v[k]);
-            bool ok = mn != 0;
-            if (s0 + sl < nsplit) ok = ok && (__float_as_uint(ml.x) | __float_as_uint(ml.y)) != 0;
-            if (__builtin_amdgcn_ballot_w64(!ok) == 0 || spin >= kMaxPolls) break;
-#ifdef X_POLLSTAT
-            if (lane == 0) atomicAdd(&g_polls[0], 1ull);
-#endif
-        }
-#ifdef X_POLLSTAT
-        if (lane == 0) atomicAdd(&g_polls[1], 1ull);
-#endif
-#else
-        if (s0 + sl < nsplit) ml = ld_dev2_at(mlb + 2 * s0, ml_lane);       // ahead of the bulk loads
-        load_partials<N>(v, head_base, lane_bytes, s0, nsplit);
-#endif
-        if (s0 == 0) {
-            float mx = ml.x;
-            for (int s = 32; s < nsplit; s += 32) {        // more than 32 splits: the other maxima
-#if X_PROTO >= 1 && !defined(X_NOZERO)
-                float2 t = none;
-                for (int spin = 0;; ++spin) {
-                    bool ok = true;
-                    if (s + sl < nsplit) {
-                        t = ld_dev2_at(mlb + 2 * s, ml_lane);
-                        ok = (__float_as_uint(t.x) | __float_as_uint(t.y)) != 0;
+            uint32_t v[N];
+            // (the lane offset as a value of the attempt: the addresses of its loads are then formed here, from the
+            // scalar base, and not kept in a pair of vector registers per load across the loop)
+            uint32_t lb = lane_bytes, mlo = ml_lane;
+            asm volatile("" : "+v"(lb), "+v"(mlo));
+            PROF_AT(pts, 8);
+            ml = ld_dev2_at(mlb, mlo);       // ahead of the bulk loads
+            load_partials<N>(v, head_base, lb, s0);
+            PROF_AT(pts, 9);
+            uint32_t mn = __float_as_uint(ml.x) | __float_as_uint(ml.y);
+            if (s0 == 0) {
+                float mx = mine ? ml.x : -INFINITY;
+                for (int s = BLOCK; s < nsplit; s += BLOCK) {        // more splits than a block holds: the other maxima
+                    float2 t = float2{-INFINITY, 0.0f};
+                    for (int spin2 = 0;; ++spin2) {
+                        bool ok = true;
+                        if (s + sl < nsplit) {
+                            t = ld_dev2_at(mlb + 2 * s, sl * 8);
+                            ok = (__float_as_uint(t.x) | __float_as_uint(t.y)) != 0;
+                        }
+                        if (__builtin_amdgcn_ballot_w64(!ok) == 0 || spin2 >= kMaxPolls) break;
                     }
-                    if (__builtin_amdgcn_ballot_w64(!ok) == 0 || spin >= kMaxPolls) break;
+                    mx = fmaxf(mx, t.x);
                 }
-                mx = fmaxf(mx, t.x);
-#else
-                if (s + sl < nsplit) mx = fmaxf(mx, ld_dev2_at(mlb + 2 * s, ml_lane).x);
-#endif
+                M = wave_max(mx);
+                Mu = (M == -INFINITY) ? 0.0f : M;
             }
-            M = wave_max(mx);
-            Mu = (M == -INFINITY) ? 0.0f : M;
+            w = mine ? __builtin_amdgcn_exp2f(ml.x - Mu) * __builtin_fabsf(ml.y) : 0.0f;
+            settle_partials<N>(v, nsplit - s0);
+#pragma unroll
+            for (int k = 0; k < N; k += 2) {
+                const float wa = lane_value(w, k), wb = lane_value(w, k + 1);
+                mn = min(mn, min(v[k], v[k + 1]));
+                e0 = __builtin_fmaf(wa, half_lo(v[k]), e0);
+                e1 = __builtin_fmaf(wa, half_hi(v[k]), e1);
+                d0 = __builtin_fmaf(wb, half_lo(v[k + 1]), d0);
+                d1 = __builtin_fmaf(wb, half_hi(v[k + 1]), d1);
+            }
+            PROF_AT(pts, 10);
+            if (__builtin_amdgcn_ballot_w64(mn == 0) == 0 || spin >= kMaxPolls) break;
+            e0 = se0;
+            e1 = se1;
+            d0 = sd0;
+            d1 = sd1;
         }
-        const float w = (s0 + sl < nsplit) ? __builtin_amdgcn_exp2f(ml.x - Mu) * ml.y : 0.0f;
         lacc += w;
-#pragma unroll
-        for (int k = 0; k < N; k += 2) {
-            const float wa = lane_value(w, k), wb = lane_value(w, k + 1);
-            e0 = __builtin_fmaf(wa, partial_lo(v[k]), e0);
-            e1 = __builtin_fmaf(wa, partial_hi(v[k]), e1);
-            d0 = __builtin_fmaf(wb, partial_lo(v[k + 1]), d0);
-            d1 = __builtin_fmaf(wb, partial_hi(v[k + 1]), d1);
-        }
-#if X_PROTO >= 1 && !defined(X_NOZERO)
-        // the records are consumed: back to "not written" for the next launch on this workspace
-        {
-            uint32_t* base = head_base + s0 * kPartialWords + lane;
-            const int cnt = nsplit - s0;
-#pragma unroll
-            for (int k = 0; k < N; ++k) {
-                if (k < cnt) st_dev1(base + k * kPartialWords, 0u);
+        // splits that sent residual words (rare: outputs of magnitude 2 or more), in ascending order; the words are set
+        // back to "not written" here, by their only reader
+        uint64_t sent = __builtin_amdgcn_ballot_w64(mine && lane < BLOCK && ml.y < 0.0f);
+        while (sent) {
+            const int s = __builtin_ctzll(sent);
+            sent &= sent - 1;
+            const float ws = lane_value(w, s);
+            uint32_t* rec = head_base + lo_words + (s0 + s) * kPartialWords;
+            uint32_t r = 0;
+            for (int spin = 0;; ++spin) {
+                r = ld_dev1_at(rec, lane_bytes);
+                if (__builtin_amdgcn_ballot_w64(r == 0) == 0 || spin >= kMaxPolls) break;
             }
-            if (lane < 32 && s0 + sl < nsplit) st_dev2(mlb + 2 * (s0 + sl), 0.0f, 0.0f);
+            e0 = __builtin_fmaf(ws, half_lo(r), e0);
+            e1 = __builtin_fmaf(ws, half_hi(r), e1);
+            st_dev1(rec + lane, 0u);
         }
-#endif
     }
     O0 = e0 + d0;
     O1 = e1 + d1;
-    // both halves of the wave hold the same 32 terms
+    // a block's terms lie in lanes 0 .. BLOCK-1 and again in the lanes behind them
     const float lrow = row_sum16(lacc);
-    L = lane_value(lrow, 0) + lane_value(lrow, 16);
+    L = BLOCK == 32 ? lane_value(lrow, 0) + lane_value(lrow, 16) : lane_value(lrow, 0);
 }
-__device__ __forceinline__ void merge_splits(uint32_t* o_part, float* ml_part, int64_t hrow,
-                                             int nsplit, int lane, float& O0, float& O1, float& M, float& L) {
+// MAXN: loads a lane may have in flight (32, or 16 in the kernels whose 16 waves leave a lane 128 registers: there
+// more than 16 splits are merged in blocks of 16, one round trip per block)
+template <int MAXN>
+__device__ __forceinline__ void merge_splits(uint32_t* o_part, uint32_t lo_words, float* ml_part, int64_t hrow,
+                                             int nsplit, int lane, float& O0, float& O1, float& M, float& L, [[maybe_unused]] unsigned long long* pts = nullptr) {
     // as many loads per lane as there are splits, rounded up to 4, 8, 16 or 32: every one of them is a round trip
     // of its own to the memory side (with 32 loads for 8 splits the 4K-token step took 0.5 us longer)
     if (nsplit <= 4) {
-        merge_splits_n<4>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<4, 32>(o_part, lo_words, ml_part, hrow, nsplit, lane, O0, O1, M, L, pts);
     } else if (nsplit <= 8) {
-        merge_splits_n<8>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<8, 32>(o_part, lo_words, ml_part, hrow, nsplit, lane, O0, O1, M, L, pts);
     } else if (nsplit <= 16) {
-        merge_splits_n<16>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<16, 32>(o_part, lo_words, ml_part, hrow, nsplit, lane, O0, O1, M, L, pts);
+    } else if constexpr (MAXN >= 32) {
+        merge_splits_n<32, 32>(o_part, lo_words, ml_part, hrow, nsplit, lane, O0, O1, M, L, pts);
     } else {
-        merge_splits_n<32>(o_part, ml_part, hrow, nsplit, lane, O0, O1, M, L);
+        merge_splits_n<16, 16>(o_part, lo_words, ml_part, hrow, nsplit, lane, O0, O1, M, L, pts);
     }
 }
 
@@ -1227,12 +1267,15 @@ __device__ __forceinline__ uint16_t to_out(float f) {
 }
 
 // Final values of one query head: lane l writes channels 2l, 2l+1 of O / L, lane 0 the natural-log LSE
-// (softmax.h:303; +inf for a row without keys).
+// (softmax.h:303; +inf for a row without keys).  One reciprocal (within a unit in the last place of 1 / L) and two
+// multiplications instead of two divisions: the wave that writes is the last thing running, and every
+// instruction of it is on the critical path.
 template <bool BF16>
 __device__ __forceinline__ void write_head(uint16_t* out_row, float* lse, int lane, float O0, float O1, float M, float L,
                                            float pshift) {
     const bool none = !(L > 0.0f);
-    const uint16_t a = to_out<BF16>(none ? 0.0f : O0 / L), b = to_out<BF16>(none ? 0.0f : O1 / L);
+    const float inv = none ? 0.0f : __builtin_amdgcn_rcpf(L);
+    const uint16_t a = to_out<BF16>(O0 * inv), b = to_out<BF16>(O1 * inv);
     if ((reinterpret_cast<uintptr_t>(out_row) & 3u) == 0) {
         reinterpret_cast<uint32_t*>(out_row)[lane] = a | (static_cast<uint32_t>(b) << 16);
     } else {
@@ -1279,13 +1322,14 @@ __device__ __forceinline__ void step_ticket(int* step_tickets, int* lengths, int
 // the new token into the window's next row, lane 0 of the wave before it sees to the length.
 template <int NW>
 __device__ __forceinline__ void step_begin(int bi, int hk, int t) {
+    constexpr int first_wave = NW - 2;
     static_assert(NW >= 2, "two waves share the append");
     const int tid = threadIdx.x;
     const int capacity = LATE_I32(capacity);
-    if (tid == (NW - 2) * 64) {
+    if (tid == first_wave * 64) {
         step_ticket(LATE_PTR(int*, step_tickets), LATE_PTR(int*, lengths), LATE_I32(hk), capacity, bi, t);
     }
-    const int lt = tid - (NW - 1) * 64;
+    const int lt = tid - (first_wave + 1) * 64;
     if (lt < 0 || lt >= 32 || step_overflows(capacity, t)) return;
     const int r = t & (kChunk - 1);
     if (lt < 16) {
@@ -1358,18 +1402,40 @@ __device__ __forceinline__ int sequence_of_position(const FwdParams& P, int p, i
 // (flash_fwd_kernel.h:1217-1298 formula) and resets the ticket.
 //
 // Dynamic LDS: [NW wave regions of UnitCfg::REGION bytes][q: 8 head rows + a zero row, 272 B apart]
-// [sM, sL: per-wave max and sum, 8 heads x NW floats each][append flag].  A wave's region is reused as its
+// [sM, sL: per-wave max and sum, 8 heads x NW floats each][append flag][tickets and slots of the 8 heads].  A wave's region is reused as its
 // V-transpose slab for fp16 tiles and as its slot of the cross-wave merge buffer (g x 128 floats <= 4 KB).
 // ---------------------------------------------------------------------------------------------
 template <int BITS, int GS, bool FEW>
 constexpr int fwd_lds_bytes() {
     using C = UnitCfg<BITS, GS, FEW>;
-    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16 + kMaxGroupHeads * 4;
+    return C::NW * C::REGION + (kMaxGroupHeads + 1) * kQRowBytes + 2 * C::NW * kMaxGroupHeads * 4 + 16 + 2 * kMaxGroupHeads * 4;
 }
 
 template <int BITS, int GS, bool BF16, bool APPEND, bool KT, bool FEW>
-__global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv_kernel(FwdParams P) {
+// (second bound: waves per SIMD the register count has to leave room for.  Two workgroups of the 8-wave kernels share
+// a compute unit when sequences differ in length, 4 waves per SIMD like the 16-wave kernels: 128 registers.  The
+// per-token-K kernel of group size 32 needs more and runs one workgroup per unit.)
+__global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64), (FEW && !(KT && GS == 32) ? 4 : 1))
+void fwd_splitkv_kernel(FwdParams P) {
     static_assert(!KT || BITS == 4, "per-token K parameters: 4 bits");
+    // The decode step with append has more parameter fields than scalar registers, and the per-token-K kernels
+    // have no vector register to spare for scalar spills: they fetch what only the window and the tail need from
+    // the kernarg segment where it is used.
+    constexpr bool kLateArgs = APPEND || KT;
+    // Everything a workgroup needs before its first loads of the stream is asked for here, in the kernel's first
+    // basic block (the fields are the head of the parameter block, kernels.h): left alone, the compiler fetches a
+    // field behind the branch that first uses it, four or five rounds of scalar loads one after the other, half a
+    // microsecond in which the memory system has nothing to do.  The rest is read where it is used.
+    asm volatile("" : : "s"(P.nsplit), "s"(P.hk), "s"(P.g), "s"(P.b), "s"(P.nsplit_magic), "s"(P.hk_magic), "s"(P.seqlen),
+                 "s"(P.reslen), "s"(P.capacity), "s"(P.res_cap), "s"(P.xcd_remap), "s"(P.seq_perm), "s"(P.seqlens),
+                 "s"(P.reslens), "s"(P.q), "s"(P.q_sb), "s"(P.q_sh), "s"(P.k_pack), "s"(P.k_params), "s"(P.v_pack),
+                 "s"(P.v_params), "s"(P.block_table), "s"(P.kpack_bh), "s"(P.kparams_bh), "s"(P.vpack_bh), "s"(P.vparams_bh),
+                 "s"(P.bt_stride), "s"(P.chunks_per_page), "s"(P.neg_scale), "s"(P.scale_log2));
+    if constexpr (!kLateArgs) {
+        asm volatile("" : : "s"(P.k_res), "s"(P.v_res), "s"(P.kres_sb), "s"(P.kres_st), "s"(P.kres_sh), "s"(P.vres_sb),
+                     "s"(P.vres_st), "s"(P.vres_sh), "s"(P.o_part), "s"(P.ml_part), "s"(P.tickets), "s"(P.out), "s"(P.out_sb),
+                     "s"(P.out_sh), "s"(P.lse), "s"(P.h));
+    }
     using C = UnitCfg<BITS, GS, FEW>;
     constexpr int NCG = C::NCG, NW = C::NW, REGION = C::REGION;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -1379,6 +1445,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     float* const sL = sM + NW * kMaxGroupHeads;
     int* const s_last = reinterpret_cast<int*>(sL + NW * kMaxGroupHeads);
     int* const s_tick = s_last + 4;       // [8] tickets drawn for the heads of the group, -1 = not yet
+    int* const s_cnt = s_tick + kMaxGroupHeads;      // [8] slot of this launch for each head of the group
     if (threadIdx.x < kMaxGroupHeads) s_tick[threadIdx.x] = -1;      // (read after the workgroup barrier of the tail)
 
     PROF_DECL;
@@ -1386,6 +1453,10 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     // Workgroups are handed to the 8 XCDs round-robin by linear id.  When the number of
     // (batch, kv-head) pairs is a multiple of 8, ids are remapped so that all splits of one pair run
     // on one XCD.
+#ifdef BITDECODE_PROF
+    asm volatile("" : : "s"(P.xcd_remap));
+    PROF(11);
+#endif
     int split, hk, bi;
     {
         const int lin = blockIdx.x;
@@ -1429,6 +1500,7 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     const int u0 = min(nU, split * ups);
     const int u1 = min(nU, u0 + ups);
     const int nT = (R + 15) / 16;
+    PROF(12);
 
     uint8_t* const region = lds + wave * REGION;
     const uint32_t region_lds = lds_addr(region);
@@ -1445,13 +1517,41 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
         qa_raw = load_untracked(q0 + (hq < g ? hq : 0) * P.q_sh);
         qb_raw = load_untracked(q0 + (hq + 4 < g ? hq + 4 : 0) * P.q_sh);
     }
+    PROF(13);
     UnitAddr<BITS, GS> A;
     if (u < u1) {
         A = unit_addr<BITS, GS, KT>(P, bi, hk, u);
+        PROF(14);
         issue_first_rows<BITS, GS, KT, FEW>(A, lane * 16, region_lds);
+        PROF(15);
         wait_then_take<C::DEPTH - 1>(qa, qb, qa_raw, qb_raw);
     } else {
         wait_then_take<0>(qa, qb, qa_raw, qb_raw);
+    }
+    if (P.nsplit > 1 && wave == 0) {
+        // Which slot of the split workspace this launch uses: a word per head next to its counter, flipped by the
+        // wave that merges the head's splits when the launch is over for that head.  Lane j fetches head j's word
+        // straight into LDS (device scope), behind the wave's first rows in its load queue (the waits of the row
+        // pipeline count it as a row until it has landed, which holds the first rows back by one at most), so that
+        // nobody ever waits for it: the tail reads it from LDS after the workgroup's barrier.
+        const int* tk;
+        if constexpr (kLateArgs) {
+            const kblock ob = karg_block<BLOCK_AT(o_part)>();       // o_part ... bits
+            tk = BLOCK_PTR(const int*, ob, o_part, tickets) +
+                 (static_cast<int64_t>(bi) * BLOCK_I32(ob, o_part, h) + hk * g) * kTicketStride + kSlotWord;
+        } else {
+            tk = P.tickets + (static_cast<int64_t>(bi) * P.h + hk * g) * kTicketStride + kSlotWord;
+        }
+        const uint64_t heads = (1ull << g) - 1;
+        uint64_t saved;
+        asm volatile("s_mov_b32 m0, %3\n\t"
+                     "s_mov_b64 %0, exec\n\t"
+                     "s_and_b64 exec, exec, %4\n\t"
+                     "global_load_lds_dword %1, %2 sc1\n\t"
+                     "s_mov_b64 exec, %0"
+                     : "=&s"(saved)
+                     : "v"(lane * (kTicketStride * 4)), "s"(tk), "s"(__builtin_amdgcn_readfirstlane(lds_addr(s_cnt))), "s"(heads)
+                     : "memory", "m0", "scc");
     }
     if (P.neg_scale) {      // softmax_scale < 0: scale_log2 holds |scale|, the sign goes into q
 #pragma unroll
@@ -1506,22 +1606,49 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
         uint16_t* slab = reinterpret_cast<uint16_t*>(region);
         const int stride = NW * P.nsplit;
         int t = wave * P.nsplit + split;   // consecutive tiles go to different workgroups
+        // (the lane index as a value of its own: what the tiles derive from it is then computed here, not carried
+        // through the unit loop from the prologue, where the q loads derive the same; the loop has no register to spare)
+        int lane_w = lane;
+        asm volatile("" : "+v"(lane_w));
         if (t < nT) {
             wait_vm<0>();                  // q rows (a wave without packed units has not waited yet)
-            const WindowSrc W = window_src<APPEND>(P, bi, hk);
+            const WindowSrc W = window_src<APPEND, kLateArgs>(P, bi, hk);
             Fp16Tile T;
-            load_fp16_tile<APPEND>(T, W, t * 16, R, lane, r_new);
+            load_fp16_tile<APPEND>(T, W, t * 16, R, lane_w, r_new);
             while (true) {
                 const int tn = t + stride;
                 const bool more = tn < nT;
-                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane, Q, lo_part, st, slab, p_shift(BITS));
+                fp16_tile<BF16, NCG>(T, P, t * 16, R, lane_w, Q, lo_part, st, slab, p_shift(BITS));
                 if (!more) break;
-                load_fp16_tile<APPEND>(T, W, tn * 16, R, lane, r_new);
+                load_fp16_tile<APPEND>(T, W, tn * 16, R, lane_w, r_new);
                 t = tn;
             }
         }
     }
 
+    // (kLateArgs: what only the tail needs is fetched here, as for the window)
+    uint16_t* out = P.out;
+    int64_t out_sb = P.out_sb, out_sh = P.out_sh;
+    float* lse_out = P.lse;
+    uint32_t* o_part = P.o_part;
+    float* ml_part = P.ml_part;
+    int* tickets = P.tickets;
+    int n_h = P.h;
+    if constexpr (kLateArgs) {
+        const kblock ob = karg_block<BLOCK_AT(o_part)>();       // o_part ... bits
+        out = BLOCK_PTR(uint16_t*, ob, o_part, out);
+        out_sb = BLOCK_I64(ob, o_part, out_sb);
+        out_sh = BLOCK_I64(ob, o_part, out_sh);
+        lse_out = BLOCK_PTR(float*, ob, o_part, lse);
+        o_part = BLOCK_PTR(uint32_t*, ob, o_part, o_part);
+        ml_part = BLOCK_PTR(float*, ob, o_part, ml_part);
+        tickets = BLOCK_PTR(int*, ob, o_part, tickets);
+        n_h = BLOCK_I32(ob, o_part, h);
+    }
+    // layout of the split workspace (kernels.h: split_slot_words): residual words behind the partial outputs of a
+    // slot, the second slot behind the first
+    const uint32_t lo_words = static_cast<uint32_t>(P.nsplit) * P.b * n_h * kPartialWords;
+    const uint32_t slot_words = (lo_words / kPartialWords * (2 * kPartialWords + 2) + 63) / 64 * 64;
     // ---- merge the waves of this workgroup through LDS (each wave's slot is its own region)
     const float lsum = st.l[0] + partner(st.l[0]);      // rows are equal; lo columns hold 0
 #pragma unroll
@@ -1552,55 +1679,42 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
     // nothing below needs another workgroup barrier (the decode step with append has one, to elect the
     // workgroup that appends).
     //
-    // Protocol between the splits of one query head (workspace: counters, partial outputs, (max, sum)
-    // pairs; all in ordinary device memory):
-    //  1. a wave writes its head's partial output and (max, sum) with device-scope write-through stores;
-    //  2. it waits until all its stores are acknowledged (s_waitcnt vmcnt(0)): they are then visible to
-    //     device-scope loads of any compute unit;
-    //  3. one lane draws a ticket from the head's counter with a device-scope atomic add (performed at the
-    //     memory side, so tickets of different compute units are totally ordered);
-    //  4. the wave whose ticket is the last one knows that every other split passed step 2 before its
-    //     step 3; it resets the counter (read again only by the next launch on this workspace) and reads
-    //     all partials with device-scope loads, which are served from the coherent level and not from a
-    //     stale line of its own caches.
-    // The asm waits are compiler barriers ("memory" clobber), so neither the stores nor the loads move
-    // across the ticket.  What would break it: a workspace in host-coherent or fine-grained memory with
-    // other scope rules, two launches in flight on one workspace, or non-zero counters at the first launch.
+    // Protocol between the splits of one query head.  Workspace (ordinary device memory, all zero before its
+    // first launch, used by one launch at a time and with one shape): a counter per head, and two slots of
+    // records per (head, split): partial output (fp16 pairs), residual words, (max, sum).  A record is "not
+    // written" while it holds a zero word; writers never store one.
+    //  * Launches alternate between the two slots: a word next to each head's counter says which one is next; it is
+    //    fetched into LDS while the workgroup streams, and flipped by the wave that ends the launch for the head.
+    //  * After the workgroup's barrier an idle wave draws the head's ticket (device-scope atomic add, performed at
+    //    the memory side, so tickets are totally ordered) while the head's own wave merges the workgroup's waves,
+    //    writes its records into the launch's slot with device-scope write-through stores, and sets its records of
+    //    the other slot back to "not written" for the next launch.  Nothing waits for the stores.
+    //  * The wave whose head drew the last ticket of the launch knows that every other split of the head is past
+    //    its barrier, so its records are written or about to be, by waves that wait for nobody.  It sets the
+    //    counter back to zero, loads all records of the slot with device-scope loads and repeats the loads of a
+    //    block while a record still reads "not written" (seldom: the ticket's round trip is longer than the way of
+    //    the stores).
+    // A record of the slot in use cannot be a leftover: its writer set it back two launches ago, after the launch
+    // that read it had ended.  What would break it: a workspace in host-coherent or fine-grained memory with other
+    // scope rules, two launches in flight on one workspace, another shape on a workspace that was not zeroed
+    // again, or a workspace that was not zero at its first launch.
     bool last = false;
     float O0 = 0.0f, O1 = 0.0f, M = -INFINITY, L = 0.0f;
-    uint16_t* out = P.out;
-    int64_t out_sb = P.out_sb, out_sh = P.out_sh;
-    float* lse_out = P.lse;
-    uint32_t* o_part = P.o_part;
-    float* ml_part = P.ml_part;
-    int* tickets = P.tickets;
-    int n_h = P.h;
-    if constexpr (APPEND) {      // as for the window: fetched late
-        const kblock ob = karg_block<BLOCK_AT(o_part)>();       // o_part ... h
-        out = BLOCK_PTR(uint16_t*, ob, o_part, out);
-        out_sb = BLOCK_I64(ob, o_part, out_sb);
-        out_sh = BLOCK_I64(ob, o_part, out_sh);
-        lse_out = BLOCK_PTR(float*, ob, o_part, lse);
-        o_part = BLOCK_PTR(uint32_t*, ob, o_part, o_part);
-        ml_part = BLOCK_PTR(float*, ob, o_part, ml_part);
-        tickets = BLOCK_PTR(int*, ob, o_part, tickets);
-        n_h = BLOCK_I32(ob, o_part, h);
-    }
-    const int hq = hk * g + wave;                                  // this wave's query head
-    const int64_t hrow = static_cast<int64_t>(bi) * n_h + hq;      // its row in [b][h] tables
-    uint16_t* const out_row = out + bi * out_sb + hq * out_sh;
-#if X_PROTO == 2
-    // The ticket of a head is drawn as soon as the workgroup is past its barrier, by a wave that has nothing else
-    // to do (wave g + j for head j), while the head's own wave merges and publishes: whoever holds the last
-    // ticket knows that every other split of the head has all its waves done and will publish without waiting
-    // for anybody.  The ticket travels through LDS.
-    const bool helpers = NW >= 2 * g && P.nsplit > 1;
-    if (helpers && wave >= g && wave < 2 * g && lane == 0) {
+    // loads in flight of the wave that merges the splits (merge_splits): 16 where the kernel is at its register limit
+    constexpr int kMergeLoads = (NW >= 16 || (KT && NW >= 12)) ? 16 : 32;
+    const bool split_run = P.nsplit > 1;
+    // With at least twice as many waves as heads in the group, wave g + j draws the ticket of head j as soon as the
+    // workgroup is past its barrier, while wave j merges the workgroup's waves and publishes: the ticket's round
+    // trip is over by the time wave j needs it.  The ticket travels through LDS (s_tick).
+    const bool helpers = NW >= 2 * g;
+    if (split_run && helpers && wave >= g && wave < 2 * g && lane == 0) {
         const int64_t hr = static_cast<int64_t>(bi) * n_h + hk * g + (wave - g);
         const int d = __hip_atomic_fetch_add(&tickets[hr * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&s_tick[wave - g], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-#endif
+    const int hq = hk * g + wave;                                  // this wave's query head
+    const int64_t hrow = static_cast<int64_t>(bi) * n_h + hq;      // its row in [b][h] tables
+    uint16_t* const out_row = out + bi * out_sb + hq * out_sh;
     if (wave < g) {
         // weights of the waves: lane (any row, w) takes wave w; the row reductions give every lane the
         // head's maximum, the weights travel to all lanes as scalars
@@ -1619,54 +1733,62 @@ __global__ __launch_bounds__((UnitCfg<BITS, GS, FEW>::NW * 64)) void fwd_splitkv
             O0 = __builtin_fmaf(a, v.x, O0);
             O1 = __builtin_fmaf(a, v.y, O1);
         }
-        if (P.nsplit == 1) {
+        if (!split_run) {
             write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
         } else {
-            st_dev1(&o_part[(hrow * P.nsplit + split) * kPartialWords + lane], pack_partial(O0, O1, L));
-#if X_PROTO >= 1
-            // (max, sum) is never two zero words: a zero maximum travels as -0
-            if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M == 0.0f ? -0.0f : M, L);
-            asm volatile("" ::: "memory");
-#else
-            if (lane == 0) st_dev2(&ml_part[(hrow * P.nsplit + split) * 2], M, L);
-            wait_vm<0>();
-#endif
+            const int par = __builtin_amdgcn_readfirstlane(s_cnt[wave]) & 1;
+            const uint32_t mine_words = par ? slot_words : 0u, other_words = par ? 0u : slot_words;
+            const int64_t rec = hrow * P.nsplit + split;
+            uint32_t* const rec_o = o_part + rec * kPartialWords + lane;
+            float* const rec_ml = ml_part + rec * 2;
+            const PartialWords W(O0, O1, L);
+            const bool sends_lo = W.large(kPartialLoFrom);      // uniform
+            if (sends_lo) st_dev1(rec_o + mine_words + lo_words, W.lo());
+            st_dev1(rec_o + mine_words, W.hi());
+            // (max, sum) is never two zero words: a zero maximum travels as -0; a negative sum says "residual words sent"
+            if (lane == 0) st_dev2(rec_ml + mine_words, M == 0.0f ? -0.0f : M, sends_lo ? -L : L);
             PROF(5);
             int drawn = 0;
-#if X_PROTO == 2
+            if (!helpers && lane == 0) {
+                drawn = __hip_atomic_fetch_add(&tickets[hrow * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            // this split's records of the other slot: "not written" again for the next launch
+            st_dev1(rec_o + other_words, 0u);
+            if (lane == 0) st_dev2(rec_ml + other_words, 0.0f, 0.0f);
             if (helpers) {
                 do {
                     drawn = __hip_atomic_load(&s_tick[wave], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 } while (drawn < 0);
-            } else if (lane == 0) {
-                drawn = __hip_atomic_fetch_add(&tickets[hrow * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-#else
-            if (lane == 0) drawn = __hip_atomic_fetch_add(&tickets[hrow * kTicketStride], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#endif
             drawn = __builtin_amdgcn_readfirstlane(drawn);
             last = drawn == P.nsplit - 1;
-            if (last && lane == 0) __hip_atomic_store(&tickets[hrow * kTicketStride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the counter starts over and the next launch takes the other slot (both read again only by the next launch)
+            if (last && lane == 0) {
+                __hip_atomic_store(&tickets[hrow * kTicketStride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&tickets[hrow * kTicketStride + kSlotWord], par ^ 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             PROF(6);
+            o_part += mine_words;
+            ml_part += mine_words;
             if constexpr (APPEND) {
                 if (wave == 0) *s_last = last;
             } else if (last) {
-                merge_splits(o_part, ml_part, hrow, P.nsplit, lane, O0, O1, M, L);
+                merge_splits<kMergeLoads>(o_part, lo_words, ml_part, hrow, P.nsplit, lane, O0, O1, M, L, PROF_TS);
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }
     }
     if constexpr (APPEND) {
-        // The workgroup whose wave 0 drew the last ticket of the group's first head appends: every other
-        // workgroup of the (batch, kv-head) has published, so none of them reads the window or the cache
+        // The workgroup whose wave 0 holds the last ticket of the group's first head appends: every other
+        // workgroup of the (batch, kv-head) is past its barrier, so none of them reads the window or the cache
         // any more.  Its last two waves store the token while the merging waves fetch the partials.
         bool appends = true;
-        if (P.nsplit > 1) {
+        if (split_run) {
             __syncthreads();
             appends = *s_last != 0;
             if (appends) step_begin<NW>(bi, hk, step_len);
             if (wave < g && last) {
-                merge_splits(o_part, ml_part, hrow, P.nsplit, lane, O0, O1, M, L);
+                merge_splits<kMergeLoads>(o_part, lo_words, ml_part, hrow, P.nsplit, lane, O0, O1, M, L, PROF_TS);
                 write_head<BF16>(out_row, lse_out ? lse_out + hrow : nullptr, lane, O0, O1, M, L, p_shift(BITS));
             }
         }
@@ -1730,15 +1852,6 @@ hipError_t launch_fwd_t(const FwdParams& P, hipStream_t stream) {
 }
 
 }  // namespace
-
-#ifdef X_POLLSTAT
-extern "C" int bitdecode_debug_polls(unsigned long long* out4) {
-    hipError_t e = hipMemcpyFromSymbol(out4, HIP_SYMBOL(g_polls), sizeof(g_polls));
-    unsigned long long z[4] = {0, 0, 0, 0};
-    if (e == hipSuccess) e = hipMemcpyToSymbol(HIP_SYMBOL(g_polls), z, sizeof(z));
-    return e != hipSuccess;
-}
-#endif
 
 #ifdef BITDECODE_PROF
 hipError_t set_prof_buffer(unsigned long long* p) {

@@ -119,9 +119,10 @@ class _on_device:
 
 
 # Split workspaces of the plain entry points, one per (device, stream, kind, batch, heads, splits): a call
-# leaves the arrival counters at the head of its workspace at zero, so the next call on the same stream can
-# take the same buffer without refilling it (calls on one stream run one after the other; two streams never
-# share a buffer).  Plans own their workspace instead: they may be replayed from anywhere.
+# leaves its workspace ready for the next call of the same shape (counters at zero, the records it used marked
+# "not written" again by the call after it), so the next call on the same stream takes the same buffer without
+# refilling it (calls on one stream run one after the other; two streams never share a buffer, and neither do
+# two shapes).  Plans own their workspace instead: they may be replayed from anywhere.
 _WORKSPACES: "dict[tuple, torch.Tensor]" = {}
 _MAX_WORKSPACES = 64
 
@@ -132,7 +133,7 @@ def _stream_workspace(device, kind: str, b: int, h: int, ns: int, nbytes: int) -
     if ws is None or ws.numel() < nbytes:
         if len(_WORKSPACES) >= _MAX_WORKSPACES:
             _WORKSPACES.pop(next(iter(_WORKSPACES)))
-        # zero-filled once: the arrival counters must be 0 before the first call
+        # zero-filled once: the whole workspace must be 0 before its first call
         ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
         _WORKSPACES[key] = ws
     return ws

@@ -100,11 +100,14 @@ typedef struct bitdecode_fwd_args {
     int64_t out_stride_b, out_stride_h;
     float* softmax_lse;        /* optional [b, h] natural-log LSE                           */
     void* workspace;           /* >= bitdecode_fwd_workspace_bytes(...) or NULL if 1 split;
-                                  ordinary device memory (hipMalloc); its first 256*b*h bytes
-                                  (one arrival counter per query head, each in a 256-byte block
-                                  of its own) must be zero before the first call and are left
-                                  zero by every call; calls that share a workspace must not
-                                  overlap in time                                            */
+                                  ordinary device memory (hipMalloc, not host-coherent or
+                                  fine-grained memory), 16-byte aligned.  ALL of it must be
+                                  zero before the first call that uses it, and again before a
+                                  call with another (b, h, num_splits) than the calls before:
+                                  the kernel tells a split's record that is written from one
+                                  that is not by its words being non-zero, and leaves the
+                                  workspace ready for the next call of the same shape.  Calls
+                                  that share a workspace must not overlap in time            */
     size_t workspace_bytes;
     int32_t b, h, h_k, d;      /* d must be 128, h % h_k == 0, h / h_k <= 8                 */
     int32_t bits, group_size, dtype;
@@ -124,10 +127,13 @@ int bitdecode_fwd(const bitdecode_fwd_args* args, void* stream);
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
  * results as bitdecode_fwd, except that `workspace` / `workspace_bytes` are ignored: partial outputs and
  * arrival counters live in an 8 MiB array inside the library's code object (one copy per GPU, held until the
- * process ends), and the call allocates nothing.  Limits: b * h <= 4096 and num_splits * b * h * 264 bytes
- * <= 7 MiB, otherwise BITDECODE_EWORKSPACE.  All calls on one GPU share that array: calls that overlap in
- * time on one GPU (two streams, two host threads) race; calls on one stream do not.  The first call on a
- * device looks up the array's address (hipGetSymbolAddress): make it outside any stream capture. */
+ * process ends), and the call allocates nothing.  Limits: b * h <= 4096 and
+ * bitdecode_fwd_workspace_bytes(b, h, num_splits) - 256 * b * h <= 7 MiB (1040 bytes per split and query
+ * head), otherwise BITDECODE_EWORKSPACE.  Every call clears the part of the array it uses with a small fill
+ * kernel in front of the decode kernel (calls of different shapes follow one another on the one array), so a
+ * call is two or three launches.  All calls on one GPU share that array: calls that overlap in time on one
+ * GPU (two streams, two host threads) race; calls on one stream do not.  The first call on a device looks up
+ * the array's address (hipGetSymbolAddress): make it outside any stream capture. */
 int bitdecode_fwd_static(const bitdecode_fwd_args* args, void* stream);
 
 /* One decode step in one launch: attend the new token together with everything held, append it, and
@@ -147,7 +153,7 @@ int bitdecode_fwd_static(const bitdecode_fwd_args* args, void* stream);
  * In `fwd`: seqlen_k, seqlens_k, res_len, res_lens and max_seqlen_k are ignored; k_res / v_res are the
  * window (written), max_res_len its capacity in tokens (at least 128); the packed cache is written;
  * workspace must hold bitdecode_fwd_append_workspace_bytes(...) bytes, required for any split count,
- * zero before the first call. */
+ * all zero before the first call and before a call with another (b, h, num_splits), as for bitdecode_fwd. */
 typedef struct bitdecode_fwd_append_args {
     bitdecode_fwd_args fwd;
     int32_t* lengths;          /* device int32[b], read and advanced                        */
@@ -174,9 +180,11 @@ int bitdecode_num_splits(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t m
 int bitdecode_num_splits_for(int32_t b, int32_t h_k, int32_t max_seqlen_k, int32_t max_res_len,
                              int32_t num_cus, int32_t bits, int32_t group_size, int32_t per_sequence_lengths);
 
-/* Workspace the split path needs: arrival counters, partial outputs (normalised, fp16) and fp32 (max, sum) pairs
- * (replaces the per-call torch::empty of out_accum / softmax_lse_accum,
- * csrc/bit_decode/decode_api.cpp:292-295). */
+/* Workspace the split path needs: a 256-byte block per query head (arrival counter and the slot the next call
+ * uses), then two slots of records that calls use in turn; a record per (query head, split) is a partial output
+ * (normalised, 64 words of two fp16), 64 residual words for outputs too large for fp16 alone, and an fp32
+ * (max, sum) pair: 256 * b * h + 2 * round_up(1040 * b * h * num_splits, 256) bytes (replaces the per-call
+ * torch::empty of out_accum / softmax_lse_accum, csrc/bit_decode/decode_api.cpp:292-295). */
 size_t bitdecode_fwd_workspace_bytes(int32_t b, int32_t h, int32_t num_splits);
 
 int bitdecode_abi_version(void);

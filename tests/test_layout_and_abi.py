@@ -277,8 +277,10 @@ def test_split_choice_and_workspace_size():
     # ... and not batches that need more than two splits to fill the machine anyway
     assert lib.bitdecode_num_splits_for(8, 8, 8192, 128, 256, 4, 128, 1) == lib.bitdecode_num_splits(8, 8, 8192, 128, 256, 4, 128) == 4
     assert lib.bitdecode_fwd_workspace_bytes(1, 32, 1) == 0
-    # one 256-byte counter block per query head + fp16 partial outputs and fp32 (max, sum) pairs per split
-    assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 32 * 256 + 32 * 32 * 66 * 4
+    # one 256-byte counter block per query head + two slots of records per split: fp16 partial outputs, as many
+    # residual words, an fp32 (max, sum) pair; a slot is a whole number of 256-byte blocks
+    assert lib.bitdecode_fwd_workspace_bytes(1, 32, 32) == 32 * 256 + 2 * 32 * 32 * 130 * 4
+    assert lib.bitdecode_fwd_workspace_bytes(1, 3, 5) == 3 * 256 + 2 * ((3 * 5 * 130 * 4 + 255) // 256 * 256)
 
 
 def test_python_entry_points_validate_before_touching_the_gpu():

@@ -27,14 +27,16 @@ def _plan(device, seed, b, h, h_k, S, R, bits, gs, ns):
                                 num_splits=ns, return_lse=True)
 
 
-def _run_static(plan, device):
-    """The plan's argument block with no workspace and fresh outputs, through bitdecode_fwd_static."""
+def _run_static(plan, device, out=None, lse=None):
+    """The plan's argument block with no workspace and fresh (or the given) outputs, through
+    bitdecode_fwd_static on the current stream."""
     from bitladder_amd import _lib
     L = _lib.lib()
     a = _lib.FwdArgs()
     ctypes.memmove(ctypes.byref(a), ctypes.byref(plan.args), ctypes.sizeof(a))
-    out = torch.full_like(plan.out, float("nan"))
-    lse = torch.full_like(plan.lse, float("nan"))
+    if out is None:
+        out = torch.full_like(plan.out, float("nan"))
+        lse = torch.full_like(plan.lse, float("nan"))
     a.out, a.softmax_lse = out.data_ptr(), lse.data_ptr()
     a.workspace, a.workspace_bytes = None, 0
     rc = L.bitdecode_fwd_static(ctypes.byref(a), torch.cuda.current_stream(device).cuda_stream)
@@ -61,6 +63,31 @@ def test_static_scratch_entry_matches_the_workspace_entry(device):
         assert torch.equal(lse, want[name][1]), name
         del out, lse
     assert torch.cuda.memory_allocated(device) == before
+
+    # The allocator of torch does not see a hipMalloc made inside the library: the device's free memory does.
+    # Outputs are allocated up front; after one warm-up call (the library looks the scratch address up once per
+    # device) a run of calls, one of them on a side stream, leaves the free memory of the device where it was.
+    outs = {name: (torch.full_like(plan.out, float("nan")), torch.full_like(plan.lse, float("nan")))
+            for name, plan in (("big", big), ("small", small))}
+    side = torch.cuda.Stream(device)
+    _run_static(big, device, *outs["big"])
+    with torch.cuda.stream(side):      # the runtime sets a stream's queue up at its first launch: not the library's doing
+        _run_static(small, device, *outs["small"])
+    side.synchronize()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(device)
+    for rep in range(6):
+        for name, plan in (("big", big), ("small", small)):
+            _run_static(plan, device, *outs[name])
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        _run_static(small, device, *outs["small"])
+    side.synchronize()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(device)
+    assert free_after == free_before, (free_before, free_after)
+    for name in outs:
+        assert torch.equal(outs[name][0], want[name][0]) and torch.equal(outs[name][1], want[name][1]), name
 
     # beyond the built-in scratch: a clear error, nothing launched
     L = _lib.lib()
