@@ -267,11 +267,11 @@ def time_steps(run_step, steps, warmup, use_graph, quantile_reps=0, steady=True,
 # read a buffer and do nothing else.  A configuration is (workgroups, threads, mode, depth, nt, pattern); see
 # bitladder_amd/csrc/probe.hip.
 PROBE_DEFAULT = [   # the configurations the sweep (--probe-sweep) found fastest at one size or another
-    (256, 1024, 0, 8, 1, 0),
-    (512, 512, 0, 8, 1, 0),
-    (1024, 256, 0, 8, 1, 0),
-    (256, 1024, 1, 4, 1, 1),
-    (512, 512, 0, 16, 1, 0),
+    (512, 256, 1, 4, 1, 0),
+    (512, 256, 1, 8, 1, 0),
+    (256, 256, 1, 8, 1, 0),
+    (256, 512, 1, 4, 1, 1),
+    (1024, 512, 1, 4, 1, 1),
 ]
 _probe_lib = None
 
@@ -367,6 +367,72 @@ def probe_sweep(args):
     return 0
 
 
+# The reference's own sweep (benchmark/bench_single_decode.ipynb:198-207, 311-316: one sequence, MHA 32 x 128,
+# S = 1024 ... 524288; and batches 2 ... 64 at S = 4096; fp16, group size 128), its published milliseconds (hardware
+# not stated, NVIDIA) as (FA2 fp16, 4-bit, 2-bit).
+REFERENCE_SWEEP_MS = {
+    ("len", 1024): (0.0430, 0.0215, 0.0174), ("len", 4096): (0.1126, 0.0440, 0.0317),
+    ("len", 32768): (0.7741, 0.2202, 0.1536), ("len", 131072): (3.0454, 0.8837, 0.6093),
+    ("len", 524288): (12.1876, 4.2557, 2.4873),
+    ("batch", 2): (0.2089, 0.0696, 0.0489), ("batch", 16): (1.8463, 0.4567, 0.2949), ("batch", 64): (7.7322, 2.3332, 1.9128),
+}
+
+
+def reference_sweep(args):
+    """The reference's sweep on this GPU (markdown on stdout): 4-bit and 2-bit decode and the library's own fp16-KV
+    path on the same shapes, every cell timed like the headline (rotated caches, one HIP graph of the steps)."""
+    from bitladder_amd import plan_fwd_kvcache_int
+    dev = torch.device("cuda:0")
+    scale = 1.0 / math.sqrt(128)
+    cases = [("len", 1, s_) for s_ in (1024, 2048, 4096, 8192, 16384, 32768, 65536, 131072, 262144, 524288)]
+    cases += [("batch", b_, 4096) for b_ in (2, 4, 8, 16, 32, 64)]
+
+    def timed(run, nbytes):
+        long_steps = nbytes > 400e6
+        return time_steps(run, 40 if long_steps else args.steps, 3 if long_steps else args.warmup, not args.no_graph,
+                          steady=not long_steps)["event_us"]
+
+    print("| sweep | b | S | 4-bit us | GB/s | frac of 8 TB/s | 2-bit us | GB/s | frac | fp16-KV us | GB/s | 4-bit x | 2-bit x "
+          "| reference ms (fp16 / 4-bit / 2-bit) | reference x |")
+    print("|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|")
+    for kind, b, S in cases:
+        cells = {}
+        for bits in (4, 2):
+            name = "sweep-%s-b%d-s%d-%dbit" % (kind, b, S, bits)
+            WORKLOADS[name] = (b, 32, 32, S, 128, bits, 128, torch.float16)
+            W = build_workload(name, 0, cpu_inputs=False, max_bufs=8)
+            n_, plans_ = W["nbuf"], W["plans"]
+            us = timed(lambda i, n_=n_, plans_=plans_: plans_[i % n_].run(), W["total_bytes"])
+            cells[bits] = (us, W["total_bytes"] / us / 1e3)
+            del W, plans_, WORKLOADS[name]
+            torch.cuda.empty_cache()
+        # the library's fp16 split-KV path over all S + 128 tokens
+        tokens = S + 128
+        fp16_bytes = b * tokens * 32 * 128 * 2 * 2 + 2 * b * 32 * 128 * 2
+        nb16 = max(2, min(8, math.ceil(320e6 / fp16_bytes)))
+        dummy = alloc_cache(b, 128, 32, 4, 128, dev)
+        fplans = []
+        src = [make_inputs_gpu(b, 32, 32, tokens, 50 + i, torch.float16, dev) for i in range(2)]
+        for i in range(nb16):
+            qd, kd, vd = src[i % 2]
+            if i >= 2:
+                kd, vd = kd.clone(), vd.clone()
+            fplans.append(plan_fwd_kvcache_int(qd, *dummy, None, scale, "k-channel", 128, 4, seqlen_k=0,
+                                               k_residual=kd, v_residual=vd))
+        us16 = timed(lambda i: fplans[i % nb16].run(), fp16_bytes)
+        del fplans, src
+        torch.cuda.empty_cache()
+        ref = REFERENCE_SWEEP_MS.get((kind, S if kind == "len" else b))
+        ref_txt = "%.4f / %.4f / %.4f" % ref if ref else "-"
+        ref_x = "%.1f / %.1f" % (ref[0] / ref[1], ref[0] / ref[2]) if ref else "-"
+        u4, g4 = cells[4]
+        u2, g2 = cells[2]
+        print("| %s | %d | %d | %.2f | %.0f | %.3f | %.2f | %.0f | %.3f | %.2f | %.0f | %.2f | %.2f | %s | %s |" % (
+            kind, b, S, u4, g4, g4 / HBM_PEAK_GBS, u2, g2, g2 / HBM_PEAK_GBS, us16, fp16_bytes / us16 / 1e3, us16 / u4,
+            us16 / u2, ref_txt, ref_x), flush=True)
+    return 0
+
+
 def cpu_baseline(q, k, v, S, R, bits, gs, scale, budget_s=20.0):
     """Reference semantics on the host cores: the torch oracle (dequantize the packed cache to
     fp32, fp32 softmax attention over [packed || residual]) timed on the same inputs."""
@@ -403,6 +469,9 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="skip the compact timing of the other BASELINE shapes")
     ap.add_argument("--probe-sweep", action="store_true",
                     help="only sweep the read probe over launch shapes and sizes and print the table")
+    ap.add_argument("--sweep", action="store_true",
+                    help="only run the reference's sweep (one sequence, MHA 32 x 128, S = 1024 ... 524288, and batches "
+                         "2 ... 64 at S = 4096; 4-bit, 2-bit and the library's fp16-KV path) and print the table")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch three plain 256 MiB device copies (a kernel of known traffic, used to scale "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -421,6 +490,8 @@ def main():
     torch.cuda.set_device(dev)
     if args.probe_sweep:
         return probe_sweep(args)
+    if args.sweep:
+        return reference_sweep(args)
     b, h, h_k, S, R, bits, gs, dtype = WORKLOADS[args.workload]
     scale = 1.0 / math.sqrt(128)
     ragged = args.workload in RAGGED
@@ -482,6 +553,8 @@ def main():
     }
     if T["quantiles"]:
         result["us_per_step_quantiles"] = T["quantiles"]
+    # (kept for the CPU leg's cross-check: the window-fill steps further down pack into the rotated caches)
+    out_gpu_first = plans[0].run().float().cpu()
 
     if not args.no_probe:
         # what the memory system alone allows: kernels that only read as many bytes as one step streams (buffers
@@ -652,8 +725,7 @@ def main():
         print("[bench] the CPU baseline leg runs on the uniform workloads only", file=sys.stderr)
     elif not args.no_cpu:
         out_cpu, t_cpu, reps = cpu_baseline(q0, k0, v0, S, R, bits, gs, scale)
-        out_gpu = plans[0].run().float().cpu()
-        torch.cuda.synchronize(dev)
+        out_gpu = out_gpu_first
         result["cpu_baseline"] = {
             "value": round(t_cpu * 1e6, 1), "unit": "us/step", "cores": torch.get_num_threads(),
             "kind": "port",

@@ -91,6 +91,39 @@ def test_c5_llama3_70b_layer_bf16_2bit(device):
     _run_config(device, 8, 64, 8, 65536, 128, 2, 128, "bf16", check_kv_heads=lambda bi: ((3 * bi + 1) % 8,))
 
 
+def test_longest_sequence_of_the_reference_sweep_524288_tokens(device):
+    """The far end of the reference's sweep (benchmark/bench_single_decode.ipynb:207: one sequence, MHA 32 x 128,
+    S = 524288, 4-bit g128).  Inputs are generated on the GPU (4 GiB per tensor); one kv head travels to the host
+    and is compared with the oracle (cache bytes bit-exact, output within tolerance), and the result must not
+    depend on the split count."""
+    from bitladder_amd import fwd_kvcache_int, kvcache_pack_int
+    b, h, h_k, S, R, bits, gs, hk = 1, 32, 32, 524288, 128, 4, 128, 21
+    g = torch.Generator(device=device).manual_seed(524288)
+    q = torch.randn((b, 1, h, 128), generator=g, device=device).half()
+    k = torch.randn((b, S + R, h_k, 128), generator=g, device=device, dtype=torch.float16)
+    v = torch.randn((b, S + R, h_k, 128), generator=g, device=device, dtype=torch.float16)
+    k[:, :, :, 5::43] *= 10.0                              # a few outlier channels, as in the other inputs
+    cache = H.alloc_cache(b, S, h_k, bits, gs, device)
+    kvcache_pack_int(k[:, :S], cache[0], cache[1], v[:, :S], cache[2], cache[3], None, None, S, "k-channel", gs, bits)
+    kw = dict(k_residual=k[:, S:], v_residual=v[:, S:])
+    outs = {ns: fwd_kvcache_int(q, *cache, None, SCALE, "k-channel", gs, bits, num_splits=ns, **kw) for ns in (0, 1, 5, 64)}
+    torch.cuda.synchronize()
+    k1 = k[:, :, hk:hk + 1].float().cpu().numpy()
+    v1 = v[:, :, hk:hk + 1].float().cpu().numpy()
+    qkv = O.quantize_kv_ref(k1[:, :S], v1[:, :S], bits, gs, "fp16")
+    # the cache tensors are containers of per-(batch, kv-head) regions: the head's region through the flat view
+    cache_np = H.cache_to_numpy(*(t.reshape(b, h_k, -1)[:, hk:hk + 1].reshape(1, t.shape[1], 1, t.shape[3]).contiguous()
+                                  for t in cache))
+    H.assert_cache_equals_oracle(cache_np, qkv)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    want, _ = O.attend_ref(q[:, :, hk:hk + 1].float().cpu().numpy(), k_hat, v_hat, SCALE, k1[:, S:], v1[:, S:])
+    errs = {ns: float(np.abs(o[:, :, hk:hk + 1].float().cpu().numpy() - want).max()) for ns, o in outs.items()}
+    spread = {ns: (o.float() - outs[0].float()).abs().max().item() for ns, o in outs.items()}
+    print("max-abs error against the oracle by split count:", errs, "; against the chosen split count:", spread)
+    assert max(errs.values()) < ATOL, errs
+    assert max(spread.values()) < 1e-3, spread
+
+
 def test_c4_ragged_batch_decode_and_append(device):
     """Batch 16, per-sequence KV length uniform in [1024, 8192] (seeded).  The packed part of
     each sequence is its length rounded down to a multiple of 128; the remainder plus 128 new
