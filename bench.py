@@ -28,11 +28,11 @@ HBM_PEAK_GBS = 8000.0
 # count; a 256 MiB device copy in the same runs reads 131085 and 262144, i.e. the fetch counter is in units of
 # 2 KiB and the write counter in KiB.
 MEASURED_TRAFFIC_BYTES = {
-    "llama3-8b-gqa-32k-4bit-g128": int(17965.51 * 2048 + 329.00 * 1024),
-    "llama2-7b-mha-4k-4bit-g128": int(9886.52 * 2048 + 89.00 * 1024),
-    "llama3-8b-gqa-128k-2bit-g64": int(41569.52 * 2048 + 329.00 * 1024),
-    "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": int(56131.44 * 2048 + 784.00 * 1024),
-    "llama3-70b-gqa-64k-2bit-g128-b8": int(150022.50 * 2048 + 784.00 * 1024),
+    "llama3-8b-gqa-32k-4bit-g128": int(17978.92 * 2048 + 619.61 * 1024),
+    "llama2-7b-mha-4k-4bit-g128": int(9901.16 * 2048 + 162.56 * 1024),
+    "llama3-8b-gqa-128k-2bit-g64": int(41589.20 * 2048 + 618.75 * 1024),
+    "llama3-8b-gqa-ragged-1k-8k-b16-4bit-g128": int(56196.71 * 2048 + 1377.33 * 1024),
+    "llama3-70b-gqa-64k-2bit-g128-b8": int(150066.51 * 2048 + 1376.00 * 1024),
 }
 
 WORKLOADS = {
