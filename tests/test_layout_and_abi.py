@@ -91,6 +91,36 @@ def test_reference_layout_converters_roundtrip_and_hand_built_group():
     assert vh[0, 1, 1, n_ - 128] == vs[0, n_, 1, 0] and vh[0, 1, 1, 128 + n_ - 128] == vz[0, n_, 1, 0]
 
 
+def test_reference_word_nibble_order_from_the_packing_statement():
+    """The reference packs four fragment elements jj .. jj+3 into one 16-bit word by or-ing val3, val2, val1, val0
+    with a 4-bit shift in between (qpack.h:283-291), so element jj + t lands in nibble t.  Restated here literally,
+    as a scalar loop over one fragment row, and compared with the converter's words.  What the statement does NOT
+    say is which token (K) or channel (V) fragment element jj + t is: the converter takes them 32 apart
+    (dequantize.h:352-375 read with the 32-row pack tile), and that reading is unpinned against a real CUDA cache."""
+    rng = np.random.default_rng(11)
+    kc = rng.integers(0, 16, (1, 128, 1, 128), dtype=np.uint8)
+    vc = rng.integers(0, 16, (1, 128, 1, 128), dtype=np.uint8)
+    z = np.zeros((1, 1, 1, 128), np.uint16)
+    zv = np.zeros((1, 128, 1, 1), np.uint16)
+    k_pack, _, v_pack, _ = L.to_reference_layout(kc, z, z, vc, zv, zv)
+
+    def pack4(vals):                       # qpack.h:283-291, literally
+        packed = 0
+        packed |= int(vals[3]) & 0xF
+        packed <<= 4
+        packed |= int(vals[2]) & 0xF
+        packed <<= 4
+        packed |= int(vals[1]) & 0xF
+        packed <<= 4
+        packed |= int(vals[0]) & 0xF
+        return packed
+
+    for p_, c_ in ((0, 0), (31, 127), (13, 77)):
+        assert int(k_pack.view(np.uint16)[0, p_, 0, c_]) == pack4([kc[0, p_ + 32 * t, 0, c_] for t in range(4)])
+    for n_, pc in ((0, 0), (127, 31), (64, 9)):
+        assert int(v_pack.view(np.uint16)[0, n_, 0, pc]) == pack4([vc[0, n_, 0, pc + 32 * t] for t in range(4)])
+
+
 def test_bf16_parameters_are_stored_as_fp16_bits():
     """A bf16 cache keeps scale/zero as fp16 bit patterns: bf16 values inside the fp16 normal range
     survive pack -> unpack unchanged, and the stored pattern is the fp16 encoding of the value."""
