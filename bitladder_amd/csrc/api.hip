@@ -7,6 +7,7 @@
 #include <stdio.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 
 #include "../../include/bitdecode.h"
@@ -39,7 +40,7 @@ constexpr size_t kStaticCounterBytes = kStaticHeads * bitdecode::kTicketStride *
 constexpr size_t kStaticScratchBytes = size_t(8) << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 // address of `scratch` on each device (the name itself is only a host-side handle)
-unsigned char* g_scratch_ptr[64] = {};
+std::atomic<unsigned char*> g_scratch_ptr[64] = {};
 
 // 16-byte stores of zero over [p, p + n16 * 16)
 __global__ void zero_fill_kernel(uint4* p, size_t n16) {
@@ -417,12 +418,12 @@ int bitdecode_fwd_static(const bitdecode_fwd_args* a, void* stream) {
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess || dev < 0 || dev >= 64)
         return fail(BITDECODE_ELAUNCH, "bitdecode_fwd_static: no current device (%s)", hipGetErrorString(e));
-    unsigned char* ptr = g_scratch_ptr[dev];
+    unsigned char* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (!ptr) {
         // once per device, with that device current: where this device keeps its copy of the array
         if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)); e != hipSuccess || !ptr)
             return fail(BITDECODE_ELAUNCH, "bitdecode_fwd_static: address of the built-in scratch: %s", hipGetErrorString(e));
-        g_scratch_ptr[dev] = ptr;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
     }
     return run_fwd(a, nullptr, stream, ptr);
 }

@@ -34,9 +34,12 @@
 //    shared by the four lanes of a head through two lane-half swaps, accumulators rescaled only
 //    when some head's max actually moved.
 //  * The waves of a workgroup merge through LDS, one wave per query head; splits merge in the
-//    same launch: that wave publishes the head's (O / sum in fp16, max, sum), draws a ticket from
-//    the head's counter, and the wave that draws the last one combines all splits of the head.
+//    same launch: that wave publishes the head's record (O / sum in fp16, max, sum) without waiting
+//    for the stores, an idle wave has meanwhile drawn a ticket from the head's counter, and the wave
+//    whose head got the last ticket loads all records of the head, checks that none of their words
+//    still reads "not written" (zero) and combines them.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -1803,14 +1806,14 @@ hipError_t launch_fwd_ttt(const FwdParams& P, hipStream_t stream) {
     constexpr int kLds = fwd_lds_bytes<BITS, GS, FEW>();
     // the dynamic-LDS limit is raised once per kernel and device (idempotent, so a race between
     // two host threads only repeats the call)
-    static bool configured[64] = {};
+    static std::atomic<bool> configured[64] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || !configured[dev]) {
+    if (dev < 0 || dev >= 64 || !configured[dev].load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT, FEW>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return e;
-        if (dev >= 0 && dev < 64) configured[dev] = true;
+        if (dev >= 0 && dev < 64) configured[dev].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((fwd_splitkv_kernel<BITS, GS, BF16, APPEND, KT, FEW>), dim3(P.nsplit * P.hk * P.b),
                        dim3(UnitCfg<BITS, GS, FEW>::NW * 64), kLds, stream, P);

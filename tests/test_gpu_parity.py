@@ -454,3 +454,57 @@ def test_plain_call_recorded_into_a_hip_graph_has_a_workspace_of_its_own(device)
         assert torch.equal(out_g, eager1), rep
         for o in outs:
             assert torch.equal(o, eager2), rep
+
+
+@pytest.mark.parametrize("bits,gs,h,h_k,ns", [(4, 128, 8, 2, 7), (2, 64, 4, 4, 32), (4, 32, 16, 2, 3)])
+def test_one_workspace_over_many_launches_with_changing_queries(device, bits, gs, h, h_k, ns):
+    """The two record slots of a split workspace are used in turn, and a launch sets its records of the other
+    slot back to "not written".  One plan (one workspace) runs 41 launches, the query rewritten in place before each:
+    every launch must give the bits that a fresh workspace gives for that query, i.e. no record of an earlier launch
+    is ever taken for one of the current launch."""
+    from bitladder_amd import plan_fwd_kvcache_int
+    b, S = 2, 128 * 33
+    q, k, v = O.make_inputs(b, h, h_k, S, 60, seed=300 + ns)
+    cache = _pack_gpu(k[:, :S], v[:, :S], bits, gs, "fp16", device, S)
+    kres, vres = H.to_dev(k[:, S:], "fp16", device), H.to_dev(v[:, S:], "fp16", device)
+    qd = H.to_dev(q, "fp16", device)
+    plan = plan_fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, k_residual=kres, v_residual=vres,
+                                num_splits=ns)
+    gen = torch.Generator(device=device).manual_seed(17)
+    for it in range(41):
+        qd.copy_(torch.randn(qd.shape, generator=gen, device=device) * (0.25 + 0.1 * (it % 9)))
+        got = plan.run().clone()
+        fresh = plan_fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, k_residual=kres,
+                                     v_residual=vres, num_splits=ns).run()
+        assert torch.equal(got, fresh), it
+
+
+def test_workspace_zeroed_again_serves_another_shape(device):
+    """The C ABI's rule for a caller-owned workspace: all zero before its first call and before a call with another
+    (b, h, num_splits).  One buffer, sized for the larger of two shapes, serves them in turn with a fill in between;
+    results equal those of workspaces of their own."""
+    import ctypes
+    from bitladder_amd import _lib, plan_fwd_kvcache_int
+    L = _lib.lib()
+
+    def plan_for(seed, b, h, h_k, S, bits, gs, ns):
+        q, k, v = O.make_inputs(b, h, h_k, S, 0, seed=seed)
+        cache = _pack_gpu(k, v, bits, gs, "fp16", device, S)
+        return plan_fwd_kvcache_int(H.to_dev(q, "fp16", device), *cache, None, SCALE, "k-channel", gs, bits,
+                                    num_splits=ns)
+
+    plans = [plan_for(410, 1, 32, 8, 128 * 64, 4, 128, 32), plan_for(411, 3, 4, 2, 128 * 10, 2, 128, 5)]
+    want = [p.run().clone() for p in plans]
+    nbytes = max(L.bitdecode_fwd_workspace_bytes(p.args.b, p.args.h, p.args.num_splits) for p in plans)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    for rep in range(3):
+        for p, w in zip(plans, want):
+            ws.zero_()
+            a = _lib.FwdArgs()
+            ctypes.memmove(ctypes.byref(a), ctypes.byref(p.args), ctypes.sizeof(a))
+            out = torch.full_like(p.out, float("nan"))
+            a.out, a.workspace, a.workspace_bytes = out.data_ptr(), ws.data_ptr(), nbytes
+            for call in range(3):      # the same shape again needs no fill
+                assert L.bitdecode_fwd(ctypes.byref(a), torch.cuda.current_stream(device).cuda_stream) == 0
+                torch.cuda.synchronize()
+                assert torch.equal(out, w), (rep, call)
