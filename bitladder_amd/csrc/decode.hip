@@ -1434,6 +1434,7 @@ void fwd_splitkv_kernel(FwdParams P) {
                  "s"(P.reslens), "s"(P.q), "s"(P.q_sb), "s"(P.q_sh), "s"(P.k_pack), "s"(P.k_params), "s"(P.v_pack),
                  "s"(P.v_params), "s"(P.block_table), "s"(P.kpack_bh), "s"(P.kparams_bh), "s"(P.vpack_bh), "s"(P.vparams_bh),
                  "s"(P.bt_stride), "s"(P.chunks_per_page), "s"(P.neg_scale), "s"(P.scale_log2));
+    if constexpr (kLateArgs && !KT) asm volatile("" : : "s"(P.tickets), "s"(P.h));      // (for the slot words below)
     if constexpr (!kLateArgs) {
         asm volatile("" : : "s"(P.k_res), "s"(P.v_res), "s"(P.kres_sb), "s"(P.kres_st), "s"(P.kres_sh), "s"(P.vres_sb),
                      "s"(P.vres_st), "s"(P.vres_sh), "s"(P.o_part), "s"(P.ml_part), "s"(P.tickets), "s"(P.out), "s"(P.out_sb),
@@ -1538,7 +1539,7 @@ void fwd_splitkv_kernel(FwdParams P) {
         // pipeline count it as a row until it has landed, which holds the first rows back by one at most), so that
         // nobody ever waits for it: the tail reads it from LDS after the workgroup's barrier.
         const int* tk;
-        if constexpr (kLateArgs) {
+        if constexpr (KT) {
             const kblock ob = karg_block<BLOCK_AT(o_part)>();       // o_part ... bits
             tk = BLOCK_PTR(const int*, ob, o_part, tickets) +
                  (static_cast<int64_t>(bi) * BLOCK_I32(ob, o_part, h) + hk * g) * kTicketStride + kSlotWord;
