@@ -459,7 +459,9 @@ def fwd_kvcache_int(q: torch.Tensor,
     (reference: bit_decode_interface.py:43-86; non-causal, no softcap, heuristic split count).
 
     q [b, 1, h, 128] fp16/bf16; returns a new tensor of the same shape.  `softmax_scale`
-    defaults to 1.0 as in the reference; callers pass 1/sqrt(d).
+    defaults to 1.0 as in the reference; callers pass 1/sqrt(d).  q [b, m, h, 128] with m > 1 rows per sequence is
+    accepted too (every row attends every key, as with the reference's fixed is_causal = False): see
+    _fwd_query_rows.
 
     Keyword-only extensions:
       seqlen_k          valid packed tokens (multiple of 128); default = capacity of the cache
@@ -469,6 +471,9 @@ def fwd_kvcache_int(q: torch.Tensor,
                         packed prefix; residual_len = valid tokens (int or int32 [b] tensor)
       num_splits        0 = choose; out = preallocated output; return_lse -> (out, lse [b, h])
     """
+    if q.dim() == 4 and q.shape[1] > 1:
+        return _fwd_query_rows(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale, quant_mode,
+                               group_size, num_bits, **kwargs)
     key = _call_key((q, k_pack, k_params, v_pack, v_params, opt_block_table),
                     (softmax_scale, quant_mode, group_size, num_bits), kwargs)
     # the split workspace comes from a per-stream cache: no allocation and no fill after the first call
@@ -476,6 +481,35 @@ def fwd_kvcache_int(q: torch.Tensor,
     return _run_kept(key, q, kwargs, lambda shared: plan_fwd_kvcache_int(
         q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale, quant_mode, group_size, num_bits,
         _stream_ws=shared, **kwargs))
+
+
+def _fwd_query_rows(q, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale, quant_mode, group_size,
+                    num_bits, out=None, return_lse=False, **kwargs):
+    """Several query rows per sequence, q [b, m, h, 128] (the reference admits them, decode_api.cpp:341, 358-368:
+    rows of the M tile; its interface fixes is_causal = False, so every row attends every key).  The kernel's
+    16 columns hold up to eight (query head, row) pairs of a kv head: the rows are folded into the head dimension,
+    8 // (h / h_k) rows per launch, and unfolded again.  Returns [b, m, h, 128] (and lse [b, m, h])."""
+    b, m, h, d = q.shape
+    h_k = v_pack.shape[2]
+    if h_k <= 0 or h % h_k or h // h_k > 8:
+        raise ValueError(f"q has {h} heads for {h_k} kv heads: need a multiple, at most 8 per kv head")
+    g = h // h_k
+    per = max(1, 8 // g)
+    res = out if out is not None else torch.empty_like(q)
+    if res.shape != q.shape or res.dtype != q.dtype or res.device != q.device:
+        raise ValueError("out must match q in shape, dtype and device")
+    lse = torch.empty((b, m, h), dtype=torch.float32, device=q.device) if return_lse else None
+    for r0 in range(0, m, per):
+        mr = min(per, m - r0)
+        # (kv head, query head in the group, row) -> one head index
+        qv = q[:, r0:r0 + mr].reshape(b, mr, h_k, g, d).permute(0, 2, 3, 1, 4).reshape(b, 1, h_k * g * mr, d).contiguous()
+        got = fwd_kvcache_int(qv, k_pack, k_params, v_pack, v_params, opt_block_table, softmax_scale, quant_mode,
+                              group_size, num_bits, return_lse=return_lse, **kwargs)
+        ov, lv = got if return_lse else (got, None)
+        res[:, r0:r0 + mr] = ov.reshape(b, h_k, g, mr, d).permute(0, 3, 1, 2, 4).reshape(b, mr, h, d)
+        if return_lse:
+            lse[:, r0:r0 + mr] = lv.reshape(b, h_k, g, mr).permute(0, 3, 1, 2).reshape(b, mr, h)
+    return (res, lse) if return_lse else res
 
 
 def plan_fwd_kvcache_int_append(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,

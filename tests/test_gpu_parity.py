@@ -508,3 +508,30 @@ def test_workspace_zeroed_again_serves_another_shape(device):
                 assert L.bitdecode_fwd(ctypes.byref(a), torch.cuda.current_stream(device).cuda_stream) == 0
                 torch.cuda.synchronize()
                 assert torch.equal(out, w), (rep, call)
+
+
+@pytest.mark.parametrize("h,h_k,m", [(8, 8, 5), (8, 2, 3), (16, 2, 2), (4, 4, 11)])
+def test_several_query_rows_per_sequence(device, h, h_k, m):
+    """q [b, m, h, d] with m > 1 (admitted by the reference, decode_api.cpp:341, 358-368; its Python interface
+    fixes is_causal = False, bit_decode_interface.py:72-84, so every row attends every key): each row must equal
+    the oracle's output for that row alone, and a call with that row alone."""
+    from bitladder_amd import fwd_kvcache_int
+    b, S, R, bits, gs = 2, 128 * 9, 37, 4, 64
+    _, k, v = O.make_inputs(b, h, h_k, S, R, seed=700 + m)
+    rng = np.random.default_rng(701 + m)
+    q = O.round_to_storage(rng.standard_normal((b, m, h, 128), dtype=np.float32), "fp16")
+    cache = _pack_gpu(k[:, :S], v[:, :S], bits, gs, "fp16", device, S)
+    kres, vres = H.to_dev(k[:, S:], "fp16", device), H.to_dev(v[:, S:], "fp16", device)
+    qd = H.to_dev(q, "fp16", device)
+    out, lse = fwd_kvcache_int(qd, *cache, None, SCALE, "k-channel", gs, bits, k_residual=kres, v_residual=vres,
+                               return_lse=True)
+    assert out.shape == qd.shape and lse.shape == (b, m, h)
+    qkv = O.quantize_kv_ref(k[:, :S], v[:, :S], bits, gs)
+    k_hat, v_hat = O.dequantize_ref(qkv)
+    for r in range(m):
+        want, want_lse = O.attend_ref(q[:, r:r + 1], k_hat, v_hat, SCALE, k[:, S:], v[:, S:])
+        assert np.abs(out[:, r:r + 1].float().cpu().numpy() - want).max() < ATOL, r
+        assert np.abs(lse[:, r].cpu().numpy() - want_lse).max() < 1e-3, r
+        alone = fwd_kvcache_int(qd[:, r:r + 1].contiguous(), *cache, None, SCALE, "k-channel", gs, bits,
+                                k_residual=kres, v_residual=vres)
+        assert (alone.float() - out[:, r:r + 1].float()).abs().max().item() < 5e-4, r
